@@ -2,7 +2,8 @@
 and slots for fixed-size per-request state.
 
 Layer groups. Every run entry of a model that keeps a cache states its need
-(:class:`KVPagesSpec` or :class:`StateSpec`). Entries with the same need form a
+(:class:`KVPagesSpec` or :class:`StateSpec`, or several of them as :class:`CacheNeeds`:
+each member joins a group by itself). Entries with the same need form a
 group. A key/value group has a page pool and, per request, a block table of its
 own: a group that reads every earlier token keeps a request's pages until the
 request ends; a group with a window gives pages back as soon as the window has
@@ -27,7 +28,7 @@ from typing import Optional, Sequence
 import numpy as np
 
 from clockwork_amd.cache.allocator import OutOfPages, PagePool
-from clockwork_amd.config.spec import KVPagesSpec, ModelSpec, PagedRowsSpec, StateSpec
+from clockwork_amd.config.spec import CacheNeeds, KVPagesSpec, ModelSpec, PagedRowsSpec, StateSpec
 
 NO_PAGE = -1
 
@@ -38,7 +39,9 @@ class GroupLayout:
 
     index: int
     need: object            # KVPagesSpec / PagedRowsSpec (pages) or StateSpec (a slot)
-    entries: tuple[int, ...]  # indices into ModelSpec.run that own a cache in this group
+    # who owns a cache in this group: indices into ModelSpec.run, or (index, member) pairs for
+    # run entries whose mixer keeps several caches (``CacheNeeds``)
+    entries: tuple
 
     @property
     def is_kv(self) -> bool:
@@ -55,19 +58,25 @@ def plan_groups(needs: Sequence[Optional[object]]) -> list[GroupLayout]:
 
     Groups come in order of first appearance, so a model's layout is stable."""
     order: list[tuple] = []
-    members: dict[tuple, list[int]] = {}
+    members: dict[tuple, list] = {}
     specs: dict[tuple, object] = {}
     for i, need in enumerate(needs):
         if need is None:
             continue
-        if not isinstance(need, (KVPagesSpec, PagedRowsSpec, StateSpec)):
-            raise TypeError(f"run entry {i}: a cache need must be KVPagesSpec, PagedRowsSpec or StateSpec, got {need!r}")
-        key = need.group_key()
-        if key not in members:
-            order.append(key)
-            members[key] = []
-            specs[key] = need
-        members[key].append(i)
+        if isinstance(need, CacheNeeds):
+            owned = [((i, m), member) for m, member in enumerate(need.needs)]
+        else:
+            owned = [(i, need)]
+        for owner, one in owned:
+            if not isinstance(one, (KVPagesSpec, PagedRowsSpec, StateSpec)):
+                raise TypeError(f"run entry {i}: a cache need must be KVPagesSpec, PagedRowsSpec, StateSpec or "
+                                f"CacheNeeds of them, got {one!r}")
+            key = one.group_key()
+            if key not in members:
+                order.append(key)
+                members[key] = []
+                specs[key] = one
+            members[key].append(owner)
     return [GroupLayout(g, specs[key], tuple(members[key])) for g, key in enumerate(order)]
 
 

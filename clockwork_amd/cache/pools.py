@@ -74,8 +74,9 @@ class CachePools:
         # tensor above, or tensors of their own)
         self.planes: list[dict] = []
         self.state: list[torch.Tensor] = []
-        self._kv_index: dict[int, tuple[int, int]] = {}     # run entry -> (paged group, row)
-        self._state_index: dict[int, tuple[int, int]] = {}  # run entry -> (state group, row)
+        # owner (a run entry, or (run entry, member) for a mixer with several caches) -> (group, row)
+        self._kv_index: dict = {}
+        self._state_index: dict = {}
         for group in groups:
             need = group.need
             if group.is_kv:
@@ -120,19 +121,29 @@ class CachePools:
     def entry_cache(self, entry: int, source: int | None = None) -> EntryCache:
         """The cache of run entry ``entry``; with ``source`` the entry reads that entry's cache."""
         owner = entry if source is None else source
+        if (owner, 0) in self._kv_index or (owner, 0) in self._state_index:
+            # a mixer with several caches: its members in the order of its ``CacheNeeds``
+            members = []
+            while (owner, len(members)) in self._kv_index or (owner, len(members)) in self._state_index:
+                members.append(self._one_cache((owner, len(members)), source is None))
+            return EntryCache(members=tuple(members), writes=source is None, block_size=self.block_size)
+        return self._one_cache(owner, source is None)
+
+    def _one_cache(self, owner, writes: bool) -> EntryCache:
         if owner in self._kv_index:
             g, row = self._kv_index[owner]
             flat = {name: t[row].reshape(-1, *t.shape[3:]) for name, t in self.planes[g].items()}
-            return EntryCache(group=g, k=flat.get("k"), v=flat.get("v"), planes=flat, writes=source is None,
+            return EntryCache(group=g, k=flat.get("k"), v=flat.get("v"), planes=flat, writes=writes,
                               block_size=self.block_size)
         if owner in self._state_index:
             g, row = self._state_index[owner]
-            return EntryCache(group=g, state=self.state[g][row], writes=source is None)
+            return EntryCache(group=g, state=self.state[g][row], writes=writes)
         return EntryCache(writes=False)
 
-    def set_fresh_state(self, entry: int, value: torch.Tensor) -> None:
+    def set_fresh_state(self, entry, value: torch.Tensor) -> None:
         """Make ``value`` what run entry ``entry``'s state begins as for every new request (a
-        part with a beginning of its own calls this once its parameters are bound)."""
+        part with a beginning of its own calls this once its parameters are bound); for a mixer
+        with several caches ``entry`` is the pair (run entry, member)."""
         g, row = self._state_index[entry]
         self.state[g][row, self.max_num_seqs + 1].copy_(value)
 

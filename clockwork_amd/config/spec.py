@@ -23,7 +23,8 @@ class ParamSpec:
         float32 stays float32 (small vectors: norm weights, biases);
       * ``"float32"`` / ``"int32"`` - always that type.
     ``init`` names the random-weights distribution: ``("normal", std)``,
-    ``("one_plus_uniform", half_width)`` or ``("zeros",)``.
+    ``("one_plus_uniform", half_width)``, ``("uniform", lo, hi)``, ``("eye_plus_normal", std)``
+    (a matrix) or ``("zeros",)``.
     """
 
     shape: tuple[int, ...]
@@ -105,6 +106,20 @@ class StateSpec:
 
 
 @dataclass(frozen=True)
+class CacheNeeds:
+    """A mixer that keeps several things between tokens (two mixers side by side in one block,
+    pages for the one and a state for the other): ``needs`` lists them, each a
+    :class:`KVPagesSpec`, :class:`PagedRowsSpec` or :class:`StateSpec`. Each joins the layer group
+    of its own kind; the mixer finds them, in this order, in ``EntryCache.members``."""
+
+    needs: tuple
+
+    def __post_init__(self):
+        if not self.needs or any(not isinstance(n, (KVPagesSpec, PagedRowsSpec, StateSpec)) for n in self.needs):
+            raise ValueError(f"CacheNeeds takes KVPagesSpec, PagedRowsSpec or StateSpec members, got {self.needs!r}")
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One block: which parts it is made of and how they are wired.
 
@@ -165,6 +180,9 @@ class ModelSpec:
     # [vocab, hidden] matrix (the embedding table itself when ``tie_embeddings`` is set)
     embedding: Any = None
     head: Any = None
+    # the longest request the model can run (a learned position table ends there); None: no limit
+    # of the model's own
+    max_positions: Optional[int] = None
     # free-form facts for reporting (bench config lines and the like), never read by parts
     info: dict = field(default_factory=dict)
 

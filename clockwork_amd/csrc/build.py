@@ -56,7 +56,9 @@ FLAGS = [
     # from the argument buffer: a short kernel's first addresses are ready that much sooner
     "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
-PLAIN_SOURCES = {"core": "core.hip", "gemm": "gemm.hip", "gemm_tile": "gemm_tile.hip", "sampling": "sampling.hip"}
+PLAIN_SOURCES = {"core": "core.hip", "gemm": "gemm.hip", "gemm_tile": "gemm_tile.hip", "sampling": "sampling.hip",
+                 "rowwise": "rowwise.hip", "sink_attention": "sink_attention.hip",
+                 "linear_recurrence": "linear_recurrence.hip"}
 ATTENTION_SOURCE = "attention.hip"
 # head sizes compiled by build_all: the tests' models, the kernel tests and the benchmark's
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 160, 224, 256)

@@ -30,6 +30,7 @@ from clockwork_amd.engine.batch import (
 )
 from clockwork_amd.parts.model import DecoderModel
 from clockwork_amd.registry import resolve_architecture
+from clockwork_amd.weights.checkpoint import CheckpointIndex
 from clockwork_amd.weights.loader import load_parameters, read_config_json
 from clockwork_amd.weights.random_init import RandomSource
 
@@ -89,6 +90,11 @@ class ModelRunner:
         self.products = ops.ProductPolicy(hip_products=cfg.model.hip_products)
         self.config_dict = config_dict if config_dict is not None else read_config_json(cfg.model.model)
         self.arch = resolve_architecture(self.config_dict)
+        if self.arch.sizes_from_checkpoint is not None and (weight_source is not None or cfg.model.weights == "checkpoint"):
+            # sizes that the design leaves to the checkpoint's tensor shapes
+            index = weight_source if weight_source is not None else CheckpointIndex(cfg.model.model)
+            self.config_dict = self.arch.sizes_from_checkpoint(
+                self.config_dict, {name: tuple(entry.shape) for name, entry in index.entries.items()})
         self.model_config = self.arch.parse_config(self.config_dict)
         self.spec = self.arch.build_spec(self.model_config)
         self.model = DecoderModel(self.spec)
@@ -138,6 +144,8 @@ class ModelRunner:
         a new request is admitted (``total_len``: pages to set aside for it in groups that keep
         every key), a known one grows. Copy-on-write copies are done here."""
         end = start + num_tokens
+        if self.spec.max_positions is not None and end > self.spec.max_positions:
+            raise ValueError(f"request {seq_id}: {end} tokens are more than the model's {self.spec.max_positions} positions")
         if not self.manager.has(seq_id):
             if start != 0:
                 raise ValueError(f"request {seq_id} is unknown but starts at position {start}")

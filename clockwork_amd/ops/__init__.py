@@ -118,6 +118,23 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_gemm_bf16_wide_partial_ok": [I, I, I, L, I],
             "cw_gemm_bf16_wide_partial": [P, L, P, P, L, I, I, I, I, I, P],
         },
+        "rowwise": {
+            "cw_embedding_pos": [P, I, P, P, P, F, P, I, I, I, I, P],
+            "cw_add_layernorm": [P, P, P, I, P, P, I, P, P, I, F, P, I, P, I, I, P],
+            "cw_gated_residual_add": [P, P, P, I, P, P, I, I, I, I, P],
+            "cw_gelu_tanh_mul": [P, P, I, I, I, P],
+            "cw_softcap": [P, L, F, P],
+            "cw_rms_mean2": [P, P, P, P, I, F, P, I, I, I, P],
+            "cw_qk_rownorm_store": [P, I, L, I, I, I, I, I, I, P, P, I, F, P, P, P, L, I, P],
+        },
+        "sink_attention": {
+            "cw_sink_attention_max_bq": [I, I, I, I],
+            "cw_sink_attention": [I, P, L, P, P, P, L, P, I, P, P, P, I, I, P, P, P, P, I, I, I, I, I, I, F, P],
+        },
+        "linear_recurrence": {
+            "cw_linear_recurrence_supported": [I, I],
+            "cw_linear_recurrence": [I, P, L, I, I, I, I, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, F, F, P],
+        },
         "sampling": {
             "cw_argmax_chunks": [I],
             "cw_argmax": [P, L, I, I, P, P, L, P],
@@ -1182,4 +1199,226 @@ def sample(logits, temperature, top_k, top_p, seeds, draws, out=None, any_top_k:
                       _ptr(out), _ptr(ws), ws.numel(), int(bool(any_top_k)) | (int(bool(any_top_p)) << 1), _stream()),
         "sample",
     )
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# Row-wise kernels of blocks with a LayerNorm, gated branches, a position table, a capped head
+def embedding_positions(table: torch.Tensor, ids: torch.Tensor, positions, pos_table, scale: float,
+                        out_resid: torch.Tensor) -> torch.Tensor:
+    """out_resid[t] = scale * table[ids[t]] + pos_table[positions[t]] in float32 ([T, H]);
+    ``pos_table`` None: no position is added."""
+    _gpu(table, ids, positions, pos_table, out_resid)
+    T = ids.numel()
+    V, H = table.shape
+    _i32(ids, T, "ids")
+    P = 0
+    if pos_table is not None:
+        _i32(positions, T, "positions")
+        _need(pos_table.dim() == 2 and pos_table.shape[1] == H and pos_table.dtype == table.dtype,
+              "the position table must be [positions, H] in the embedding table's type")
+        P = pos_table.shape[0]
+    _need(out_resid.dtype == torch.float32 and tuple(out_resid.shape) == (T, H), "residual must be [T, H] float32")
+    _check(_load("rowwise").cw_embedding_pos(_ptr(table), dtype_code(table.dtype), _ptr(ids), _ptr(positions),
+                                             _ptr(pos_table), float(scale), _ptr(out_resid), T, H, V, P, _stream()),
+           "embedding_positions")
+    return out_resid
+
+
+class GatedBranches:
+    """What a block with gated branches still has to add to the residual stream:
+    sigmoid(z[:, :H] + zb[:H]) * a + sigmoid(z[:, H:] + zb[H:]) * b. ``z`` [T, H or 2H] are the
+    gates' products, ``zb`` their biases (or None); without ``z`` the branches count as they are;
+    ``b`` may be None. A norm that ``accepts_gated`` adds it inside its own kernel."""
+
+    __slots__ = ("z", "zb", "a", "b")
+
+    def __init__(self, z, zb, a, b=None) -> None:
+        self.z, self.zb, self.a, self.b = z, zb, a, b
+
+    @property
+    def shape(self):
+        return self.a.shape
+
+    def check(self, T: int, H: int, dtype) -> None:
+        _gpu(self.z, self.zb, self.a, self.b)
+        _need(tuple(self.a.shape) == (T, H) and self.a.dtype == dtype, "a gated branch must be [T, H] in the activation type")
+        if self.b is not None:
+            _need(tuple(self.b.shape) == (T, H) and self.b.dtype == dtype, "a gated branch must be [T, H] in the activation type")
+        if self.z is not None:
+            cols = 2 * H if self.b is not None else H
+            _need(self.z.dim() == 2 and self.z.shape[0] == T and self.z.shape[1] in (cols, 2 * H) and self.z.dtype == dtype,
+                  f"the gates' products must be [T, {cols}] in the activation type")
+            if self.zb is not None:
+                _need(self.zb.numel() == self.z.shape[1], "the gates' biases must match their products")
+        else:
+            _need(self.zb is None, "gate biases without gates")
+
+    def args(self):
+        return (_ptr(self.z), _ptr(self.zb), dtype_code(self.zb.dtype) if self.zb is not None else 0, _ptr(self.a),
+                _ptr(self.b), int(self.z.shape[1]) if self.z is not None else 0)
+
+
+def gated_residual_add(resid: torch.Tensor, pending: GatedBranches) -> torch.Tensor:
+    """resid += the gated branches' value (float32)."""
+    _gpu(resid)
+    T, H = resid.shape
+    _need(resid.dtype == torch.float32, "the residual stream is float32")
+    pending.check(T, H, pending.a.dtype)
+    _check(_load("rowwise").cw_gated_residual_add(_ptr(resid), *pending.args(), dtype_code(pending.a.dtype), T, H, _stream()),
+           "gated_residual_add")
+    return resid
+
+
+def add_layernorm(resid, pending, weight, bias, eps: float, out, rows=None) -> torch.Tensor:
+    """resid += pending (a :class:`GatedBranches` or None), out = LayerNorm(resid) * weight + bias
+    with float32 statistics (the mean, then the mean of the squared deviations); with ``rows``
+    only those rows are normed into out[i] and resid is left alone."""
+    _gpu(resid, weight, bias, out, rows)
+    T, H = resid.shape
+    _need(resid.dtype == torch.float32, "the residual stream is float32")
+    n = T if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, n, "rows")
+    _need(tuple(out.shape) == (n, H), f"out must be [{n}, {H}]")
+    _need(weight.numel() == H and (bias is None or (bias.numel() == H and bias.dtype == weight.dtype)),
+          "norm weight and bias must have the row's size and one type")
+    if pending is not None:
+        pending.check(T, H, out.dtype)
+        args = pending.args()
+    else:
+        args = (None, None, 0, None, None, 0)
+    _check(_load("rowwise").cw_add_layernorm(_ptr(resid), *args, _ptr(weight), _ptr(bias), dtype_code(weight.dtype),
+                                             float(eps), _ptr(out), dtype_code(out.dtype), _ptr(rows), n, H, _stream()),
+           "add_layernorm")
+    return out
+
+
+def gelu_tanh_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, i] = gelu_tanh(gate_up[t, i]) * gate_up[t, I + i]."""
+    _gpu(gate_up, out)
+    T, two_i = gate_up.shape
+    _need(two_i % 2 == 0 and tuple(out.shape) == (T, two_i // 2) and out.dtype == gate_up.dtype, "gelu_tanh_mul shapes")
+    _check(_load("rowwise").cw_gelu_tanh_mul(_ptr(gate_up), _ptr(out), dtype_code(out.dtype), T, two_i // 2, _stream()),
+           "gelu_tanh_mul")
+    return out
+
+
+def softcap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits <- cap * tanh(logits / cap), in place (float32)."""
+    _gpu(logits)
+    _need(logits.dtype == torch.float32 and cap > 0, "the cap takes float32 logits and a positive cap")
+    _check(_load("rowwise").cw_softcap(_ptr(logits), logits.numel(), float(cap), _stream()), "softcap")
+    return logits
+
+
+def rms_mean2(a: torch.Tensor, b, wa: torch.Tensor, wb, eps: float) -> torch.Tensor:
+    """(rms(a) * wa + rms(b) * wb) / 2 row by row, rms(x) = x / sqrt(mean(x^2) + eps) in float32;
+    ``b`` None: rms(a) * wa."""
+    _gpu(a, b, wa, wb)
+    T, H = a.shape
+    _need(wa.numel() == H, "norm weight has the wrong size")
+    if b is not None:
+        _need(b.shape == a.shape and b.dtype == a.dtype and wb is not None and wb.numel() == H and wb.dtype == wa.dtype,
+              "the second row and its weight must match the first")
+    out = torch.empty_like(a)
+    _check(_load("rowwise").cw_rms_mean2(_ptr(a), _ptr(b), _ptr(wa), _ptr(wb), dtype_code(wa.dtype), float(eps), _ptr(out),
+                                         dtype_code(a.dtype), T, H, _stream()), "rms_mean2")
+    return out
+
+
+def qk_rownorm_store(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, nq: int, nk: int, nv: int, q_weight, k_weight,
+                     eps: float, slots, k_cache, v_cache) -> None:
+    """Rows of ``proj`` [T, width] hold a token's query, key and value projections at the given
+    columns: the query projection is RMS-normed as one vector (all heads at once) with
+    ``q_weight`` and rewritten in place, the key projection likewise into the cache row
+    ``k_cache[slots[t]]``, the values are copied to ``v_cache[slots[t]]``. Caches are flat
+    [rows, nk] and [rows, nv] (any trailing shape of that many elements); a negative slot writes
+    nothing; ``slots`` None: queries only."""
+    _gpu(proj, q_weight, k_weight, slots, k_cache, v_cache)
+    T, width = proj.shape
+    cache_rows = 0
+    if slots is not None:
+        _i32(slots, T, "slots")
+        _need(k_cache is not None and v_cache is not None and k_cache.dtype == proj.dtype and v_cache.dtype == proj.dtype,
+              "the cache must be there and of the activations' type")
+        _need(k_cache.numel() % nk == 0 and v_cache.numel() % nv == 0 and k_cache.numel() // nk == v_cache.numel() // nv,
+              "key and value planes must hold the same number of rows")
+        cache_rows = k_cache.numel() // nk
+    for w, n in ((q_weight, nq), (k_weight, nk)):
+        _need(w is None or w.numel() == n, "a projection's norm weight must have the projection's size")
+    if q_weight is not None and k_weight is not None:
+        _need(q_weight.dtype == k_weight.dtype, "the two norm weights must be of one type")
+    wt = q_weight if q_weight is not None else k_weight
+    _check(_load("rowwise").cw_qk_rownorm_store(
+        _ptr(proj), dtype_code(proj.dtype), width, q_off, k_off, v_off, nq, nk, nv, _ptr(q_weight), _ptr(k_weight),
+        dtype_code(wt.dtype) if wt is not None else 0, float(eps), _ptr(slots), _ptr(k_cache), _ptr(v_cache), cache_rows, T,
+        _stream()), "qk_rownorm_store")
+
+
+# ---------------------------------------------------------------------------------------------
+def sink_attention_max_run(heads: int, kv_heads: int, dim: int, vdim: int) -> int:
+    """The most query tokens a workgroup of the sink-attention kernel takes for this geometry
+    (0: the geometry is beyond the kernel)."""
+    return int(_load("sink_attention").cw_sink_attention_max_bq(heads, kv_heads, dim, vdim))
+
+
+def sink_attention(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int, run: int,
+                   r1, r2, sink, talk, heads: int, kv_heads: int, dim: int, vdim: int, block_size: int, window: int,
+                   scale: float) -> None:
+    """Attention of the step's queries (``q`` [T, q_stride], a token's heads * dim query elements
+    first) over paged keys [rows, kv_heads, dim] and values [rows, kv_heads, vdim], into ``out``
+    [T, heads * vdim]. Options (each None: off): ``r1``/``r2`` float32 [heads], the score loses
+    r1 * log(1 + r2 * distance); ``sink`` float32 [heads], exp(sink) joins the softmax
+    denominator; ``talk`` float32 [heads, heads], the normalised weights are mixed across heads.
+    ``items`` int32 [n_items, 4]: (request, first token, tokens <= run, 0)."""
+    _gpu(q, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, r1, r2, sink, talk)
+    T = q.shape[0]
+    _need(q.dim() == 2 and q.shape[1] == q_stride and heads * dim <= q_stride, "q must be [T, q_stride] with the query heads first")
+    _need(tuple(out.shape) == (T, heads * vdim) and out.dtype == q.dtype, "out must be [T, heads * vdim]")
+    _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "cache and activations differ in type")
+    _need(tuple(k_cache.shape[-2:]) == (kv_heads, dim) and tuple(v_cache.shape[-2:]) == (kv_heads, vdim),
+          "the planes must be [..., kv_heads, dim] and [..., kv_heads, vdim]")
+    rows = k_cache.numel() // (kv_heads * dim)
+    _need(rows == v_cache.numel() // (kv_heads * vdim), "key and value planes must hold the same number of rows")
+    R = ctx_lens.numel()
+    _i32(ctx_lens, R, "ctx_lens")
+    _i32(cu_q, R + 1, "cu_q")
+    _i32(items, 4 * n_items, "items")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= R, "block tables must be int32 [R, width]")
+    for t, n, what in ((r1, heads, "r1"), (r2, heads, "r2"), (sink, heads, "sink"), (talk, heads * heads, "talk")):
+        _need(t is None or (t.dtype == torch.float32 and t.numel() == n), f"{what} must be float32 with {n} elements")
+    _need((r1 is None) == (r2 is None), "the distance bias takes r1 and r2 together")
+    _check(_load("sink_attention").cw_sink_attention(
+        dtype_code(q.dtype), _ptr(q), q_stride, _ptr(out), _ptr(k_cache), _ptr(v_cache), rows, _ptr(block_tables),
+        block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, run, _ptr(r1), _ptr(r2), _ptr(sink),
+        _ptr(talk), heads, kv_heads, dim, vdim, block_size, int(window), float(scale), _stream()), "sink_attention")
+
+
+def linear_recurrence_supported(dim: int, vdim: int) -> bool:
+    return bool(_load("linear_recurrence").cw_linear_recurrence_supported(dim, vdim))
+
+
+def linear_recurrence(proj, q_off: int, k_off: int, v_off: int, g_off: int, u_off: int, a2, a2_bias, norm_weight, state,
+                      state_slots, cu_q, n_requests: int, heads: int, dim: int, vdim: int, q_scale: float, tau: float,
+                      eps: float) -> torch.Tensor:
+    """The decayed recurrence S <- diag(a) S + k v^T, o = S^T (q_scale q) over the step's tokens,
+    request by request from each request's slot of ``state`` (float32 [slots, heads, dim, vdim],
+    updated in place). Rows of ``proj`` hold q, k (heads * dim), v, the output gate (heads * vdim;
+    ``g_off`` < 0: none) and the decay's low-rank input (``a2`` [heads * dim, rank] maps it to
+    z; a = sigmoid(z + bias)^(1/tau)). The outputs are RMS-normed over vdim with ``norm_weight``
+    (None: not) and multiplied by silu(gate). Returns [T, heads * vdim]."""
+    _gpu(proj, a2, a2_bias, norm_weight, state, state_slots, cu_q)
+    T, width = proj.shape
+    _need(a2.dim() == 2 and a2.shape[0] == heads * dim and a2.dtype == proj.dtype, "a2 must be [heads * dim, rank] in the activation type")
+    _need(a2_bias is None or (a2_bias.dtype == torch.float32 and a2_bias.numel() == heads * dim), "the decay bias must be float32 [heads * dim]")
+    _need(norm_weight is None or (norm_weight.dtype == torch.float32 and norm_weight.numel() == vdim), "the norm weight must be float32 [vdim]")
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, dim, vdim), "the state must be float32 [slots, heads, dim, vdim]")
+    _i32(state_slots, n_requests, "state_slots")
+    _i32(cu_q, n_requests + 1, "cu_q")
+    out = torch.empty((T, heads * vdim), dtype=proj.dtype, device=proj.device)
+    _check(_load("linear_recurrence").cw_linear_recurrence(
+        dtype_code(proj.dtype), _ptr(proj), width, q_off, k_off, v_off, g_off, u_off, _ptr(a2), _ptr(a2_bias),
+        _ptr(norm_weight), _ptr(state), state.shape[0], _ptr(state_slots), _ptr(cu_q), _ptr(out), n_requests, heads, dim,
+        vdim, a2.shape[1], float(q_scale), 1.0 / float(tau), float(eps), _stream()), "linear_recurrence")
     return out

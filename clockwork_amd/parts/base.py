@@ -24,7 +24,7 @@ Roles and their run methods:
                  activation type. With ``rows`` only those rows are produced and
                  ``resid`` is left untouched.
 * mixer:         ``forward(x, ctx, cache) -> y`` with x, y [T, H] in the activation
-                 type (y may be an ``ops.PartialSums``: it only ever goes to a norm); ``cache_need()`` returns a KVPagesSpec, a StateSpec or None.
+                 type (y may be an ``ops.PartialSums``: it only ever goes to a norm); ``cache_need()`` returns a KVPagesSpec, a PagedRowsSpec, a StateSpec, a CacheNeeds of several, or None.
                  ``cache`` is the run entry's :class:`EntryCache`.
 * feed-forward:  ``forward(x, ctx) -> y``.
 * position enc.: used by a mixer, not by the block; the attention mixer expects
@@ -102,3 +102,6 @@ class EntryCache:
     state: Any = None
     writes: bool = True
     block_size: int = 0
+    # a mixer that keeps several caches (``CacheNeeds``) finds one EntryCache per need here, in
+    # the order of its needs, and hands each to the part it belongs to
+    members: Any = None

@@ -44,3 +44,71 @@ class PreNormBlock:
             return ops.PendingPair(a, self.feed_forward.forward(lazy(resid, a), ctx))
         x = self.ffn_norm.forward(resid, a)
         return self.feed_forward.forward(x, ctx)
+
+
+class BranchGate:
+    """Sigmoid gates on a block's branches (``BranchGateSpec``): one product of the block's normed
+    input with all gates' matrices; the sigmoids and the biases are applied where the branches are
+    added to the residual stream (``ops.GatedBranches``)."""
+
+    graph_safe = True
+
+    def __init__(self, spec) -> None:
+        self.spec = spec
+
+    def param_specs(self):
+        from clockwork_amd.config.spec import ParamSpec
+
+        n = self.spec.branches * self.spec.hidden_size
+        return {"weight": ParamSpec((n, self.spec.hidden_size)),
+                "bias": ParamSpec((n,), precision="float32", init=("normal", 0.5))}
+
+    def cache_need(self):
+        return None
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None)]
+
+    def bind(self, params, device, dtype) -> None:
+        self.weight, self.bias = params["weight"], params["bias"]
+
+    def forward(self, x, ctx):
+        """The gates' products [T, branches * hidden] (before bias and sigmoid)."""
+        return ops.linear(x, self.weight, policy=getattr(ctx, "products", None))
+
+
+class ParallelBlock:
+    """One norm, mixer and feed-forward side by side on its output:
+    x = x + g1 * mixer(norm(x)) + g2 * ffn(norm(x)), with g = sigmoid(W norm(x) + c) from the
+    block's ``gate`` part, or 1 without one; the feed-forward may be absent.
+
+    The residual stream is float32. The block hands its branches on unadded, as
+    ``ops.GatedBranches``, when the norm that comes next adds them inside its own kernel
+    (``accepts_gated``); else it adds them itself with one kernel."""
+
+    def __init__(self, mixer, mixer_norm, feed_forward=None, gate=None) -> None:
+        self.mixer, self.mixer_norm, self.feed_forward, self.gate = mixer, mixer_norm, feed_forward, gate
+        if gate is not None and gate.spec.branches != (2 if feed_forward is not None else 1):
+            raise ValueError("a block's gate needs one set of gates per branch")
+
+    def parts(self) -> dict:
+        parts = {"mixer": self.mixer, "mixer_norm": self.mixer_norm}
+        if self.feed_forward is not None:
+            parts["feed_forward"] = self.feed_forward
+        if self.gate is not None:
+            parts["gate"] = self.gate
+        return parts
+
+    def first_norm(self):
+        return self.mixer_norm
+
+    def forward(self, resid, delta, ctx, cache):
+        x = self.mixer_norm.forward(resid, delta)
+        a = self.mixer.forward(x, ctx, cache)
+        b = self.feed_forward.forward(x, ctx) if self.feed_forward is not None else None
+        z = self.gate.forward(x, ctx) if self.gate is not None else None
+        pending = ops.GatedBranches(z, self.gate.bias if self.gate is not None else None, a, b)
+        if getattr(ctx, "next_norm_accepts_gated", False):
+            return pending
+        ops.gated_residual_add(resid, pending)
+        return None

@@ -18,7 +18,7 @@ import torch
 from clockwork_amd import ops
 from clockwork_amd.config.spec import ParamSpec
 from clockwork_amd.parts.base import Part
-from clockwork_amd.parts.specs import LinearHeadSpec, TokenEmbeddingSpec
+from clockwork_amd.parts.specs import LinearHeadSpec, PositionTableEmbeddingSpec, TokenEmbeddingSpec
 
 
 class TokenEmbedding(Part):
@@ -40,6 +40,37 @@ class TokenEmbedding(Part):
     def forward(self, ctx) -> torch.Tensor:
         resid = torch.empty((ctx.num_tokens, self.spec.hidden_size), dtype=torch.float32, device=self.device)
         return ops.embedding(self.weight, ctx.token_ids, resid)
+
+
+class PositionTableEmbedding(Part):
+    """scale * table[id] + positions[p] in float32, p the token's index in its request
+    (``ctx.positions``); a tied head gets the table itself, without the scale."""
+
+    graph_safe = True
+
+    def __init__(self, spec: PositionTableEmbeddingSpec) -> None:
+        self.spec = spec
+
+    def param_specs(self):
+        specs = {"weight": ParamSpec((self.spec.vocab_size, self.spec.hidden_size))}
+        if self.spec.max_positions is not None:
+            specs["positions"] = ParamSpec((self.spec.max_positions, self.spec.hidden_size))
+        return specs
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None)]
+
+    def bind(self, params, device, dtype) -> None:
+        self.weight = params["weight"]
+        self.position_table = params.get("positions")
+        self.device = device
+
+    def table(self) -> torch.Tensor:
+        return self.weight
+
+    def forward(self, ctx) -> torch.Tensor:
+        resid = torch.empty((ctx.num_tokens, self.spec.hidden_size), dtype=torch.float32, device=self.device)
+        return ops.embedding_positions(self.weight, ctx.token_ids, ctx.positions, self.position_table, self.spec.scale, resid)
 
 
 class LinearHead(Part):
@@ -82,4 +113,10 @@ class LinearHead(Part):
         return [self.weight]
 
     def forward(self, rows: torch.Tensor, ctx) -> torch.Tensor:
-        return ops.linear(rows, self.weight, out_dtype=torch.float32, policy=getattr(ctx, "products", None))
+        logits = ops.linear(rows, self.weight, out_dtype=torch.float32, policy=getattr(ctx, "products", None))
+        if self.spec.softcap is not None:
+            ops.softcap_(logits, self.spec.softcap)
+        return logits
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None)] if self.spec.softcap is not None else []

@@ -35,3 +35,33 @@ class SwiGLU(Part):
     def forward(self, x, ctx) -> torch.Tensor:
         policy = getattr(ctx, "products", None)
         return ops.linear(ops.linear_swiglu(x, self.gate_up, policy=policy), self.down, partial_ok=True, policy=policy)
+
+
+class GatedMLP(Part):
+    """down(act(gate(x)) * up(x)) with the activation the spec names. "silu" takes the fused
+    kernels of :class:`SwiGLU`; "gelu_tanh" runs the gate/up product, one kernel for
+    gelu_tanh(gate) * up in float32, and the down product."""
+
+    graph_safe = True
+
+    def __init__(self, spec) -> None:
+        self.spec = spec
+
+    def param_specs(self):
+        H, I = self.spec.hidden_size, self.spec.intermediate_size
+        return {"gate_up_weight": ParamSpec((2 * I, H)), "down_weight": ParamSpec((H, I))}
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None)] if self.spec.activation != "silu" else []
+
+    def bind(self, params, device, dtype) -> None:
+        self.gate_up = params["gate_up_weight"]
+        self.down = params["down_weight"]
+
+    def forward(self, x, ctx) -> torch.Tensor:
+        policy = getattr(ctx, "products", None)
+        if self.spec.activation == "silu":
+            return ops.linear(ops.linear_swiglu(x, self.gate_up, policy=policy), self.down, policy=policy)
+        gate_up = ops.linear(x, self.gate_up, policy=policy)
+        inner = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
+        return ops.linear(ops.gelu_tanh_mul(gate_up, inner), self.down, policy=policy)

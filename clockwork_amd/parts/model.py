@@ -156,6 +156,7 @@ class DecoderModel:
             else:
                 nxt = self.final_norm
             ctx.next_norm_accepts_pending = bool(getattr(nxt, "accepts_pending", False))
+            ctx.next_norm_accepts_gated = bool(getattr(nxt, "accepts_gated", False))
             delta = self.layers[entry.layer].forward(resid, delta, ctx, caches[i])
         if ctx.num_logit_rows == 0:
             return None

@@ -33,3 +33,38 @@ class RMSNorm(Part):
         """The norm of resid + delta for a consumer that computes it inside its own kernel; the
         residual is not updated, so ``delta`` has to reach the next norm as well."""
         return ops.LazyAddNorm(resid, delta, self.weight, self.spec.eps, self.dtype)
+
+
+class LayerNorm(Part):
+    """LayerNorm with weight and bias, fused with the residual add. The statistics are float32:
+    the mean first, then the mean of the squared deviations. What it can add before norming is a
+    block's gated branches (``ops.GatedBranches``): the gates' sigmoids are made inside the kernel."""
+
+    graph_safe = True
+    accepts_gated = True
+
+    def __init__(self, spec) -> None:
+        self.spec = spec
+
+    def param_specs(self):
+        specs = {"weight": ParamSpec((self.spec.size,), precision="stored", init=("one_plus_uniform", 0.1))}
+        if self.spec.bias:
+            specs["bias"] = ParamSpec((self.spec.size,), precision="stored", init=("normal", 0.02))
+        return specs
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None)]
+
+    def bind(self, params, device, dtype) -> None:
+        self.weight = params["weight"]
+        self.bias = params.get("bias")
+        if self.bias is not None and self.bias.dtype != self.weight.dtype:
+            self.bias = self.bias.to(self.weight.dtype)
+        self.dtype = dtype
+
+    def forward(self, resid: torch.Tensor, delta, rows=None) -> torch.Tensor:
+        if delta is not None and not isinstance(delta, ops.GatedBranches):
+            delta = ops.GatedBranches(None, None, delta if not isinstance(delta, ops.PartialSums) else delta.sum(self.dtype))
+        n = resid.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.spec.size), dtype=self.dtype, device=resid.device)
+        return ops.add_layernorm(resid, delta, self.weight, self.bias, self.spec.eps, out, rows)

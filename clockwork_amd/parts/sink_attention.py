@@ -1,0 +1,113 @@
+"""Windowed softmax attention with whole-projection query/key norms, a bias on the distance, a
+sink in the softmax denominator and a mixing of the weights across heads (``SinkAttentionSpec``).
+
+Steps: one fused q/k/v product; one kernel norms the query and key projections (float32
+statistics) and writes keys and values to their pages, so every token of the step is in the
+cache before any query reads it; the attention kernel reads the pages through the block table,
+prompt portions and single tokens in the same launch; output product. Keys and values have
+widths of their own, so the cache is two planes of a ``PagedRowsSpec``.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from clockwork_amd import ops
+from clockwork_amd.config.spec import PagedRowsSpec, ParamSpec
+from clockwork_amd.parts.base import EntryCache, Part
+from clockwork_amd.parts.specs import SinkAttentionSpec
+
+
+def query_runs(ctx, run: int):
+    """The step's work items for a kernel whose workgroups take up to ``run`` consecutive tokens
+    of one request with all heads: (request, first token, tokens, 0) each, uploaded once a step
+    and kept in ``ctx.plans``. Returns (device int32 array, number of items)."""
+    key = ("query runs", run)
+    plan = ctx.plans.get(key)
+    if plan is None:
+        items = []
+        for r, q_len in enumerate(ctx.h_q_lens):
+            tok0 = np.arange(0, q_len, run, dtype=np.int32)
+            rows = np.zeros((tok0.size, 4), dtype=np.int32)
+            rows[:, 0] = r
+            rows[:, 1] = tok0
+            rows[:, 2] = np.minimum(run, q_len - tok0)
+            items.append(rows.reshape(-1))
+        flat = np.concatenate(items) if items else np.zeros(0, dtype=np.int32)
+        (device_items,) = ctx.upload([flat])
+        plan = ctx.plans[key] = (device_items, len(flat) // 4)
+    return plan
+
+
+class SinkAttention(Part):
+    graph_safe = True
+
+    def __init__(self, spec: SinkAttentionSpec) -> None:
+        self.spec = spec
+        self.q_width = spec.num_heads * spec.key_dim
+        self.k_width = spec.num_kv_heads * spec.key_dim
+        self.v_width = spec.num_kv_heads * spec.value_dim
+
+    def param_specs(self):
+        s = self.spec
+        specs = {
+            "qkv_weight": ParamSpec((self.q_width + self.k_width + self.v_width, s.hidden_size)),
+            "out_weight": ParamSpec((s.hidden_size, s.num_heads * s.value_dim)),
+        }
+        if s.qk_norm == "projection":
+            specs["q_norm"] = ParamSpec((self.q_width,), precision="float32", init=("one_plus_uniform", 0.1))
+            specs["k_norm"] = ParamSpec((self.k_width,), precision="float32", init=("one_plus_uniform", 0.1))
+        if s.distance_bias:
+            specs["r1"] = ParamSpec((s.num_heads,), precision="float32", init=("uniform", 0.0, 1.0))
+            specs["r2"] = ParamSpec((s.num_heads,), precision="float32", init=("uniform", 0.0, 1.0))
+        if s.sink:
+            specs["sink"] = ParamSpec((s.num_heads,), precision="float32", init=("normal", 1.0))
+        if s.talking_heads:
+            specs["talk"] = ParamSpec((s.num_heads, s.num_heads), precision="float32", init=("eye_plus_normal", 0.2))
+        return specs
+
+    def cache_need(self):
+        s = self.spec
+        return PagedRowsSpec((("k", (s.num_kv_heads, s.key_dim)), ("v", (s.num_kv_heads, s.value_dim))), window=s.window)
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None), ("sink_attention", None)]
+
+    def bind(self, params, device, dtype) -> None:
+        s = self.spec
+        self.qkv_weight = params["qkv_weight"]
+        self.out_weight = params["out_weight"]
+        self.q_norm, self.k_norm = params.get("q_norm"), params.get("k_norm")
+        self.r1, self.r2 = params.get("r1"), params.get("r2")
+        self.sink, self.talk = params.get("sink"), params.get("talk")
+        self.dtype = dtype
+        self.run = ops.sink_attention_max_run(s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim)
+        if self.run < 1:
+            raise ValueError(
+                f"attention with {s.num_heads} heads of {s.key_dim} / {s.value_dim} elements over {s.num_kv_heads} "
+                "key/value heads is beyond the sink-attention kernel (heads * value_dim up to 8192, 150 KB of LDS)")
+
+    def _runs(self, ctx):
+        # single tokens only: a run is one token; else the most the kernel takes
+        run = 1 if all(q == 1 for q in ctx.h_q_lens) else self.run
+        return run, query_runs(ctx, run)
+
+    def prepare(self, ctx) -> None:
+        self._runs(ctx)
+
+    def forward(self, x: torch.Tensor, ctx, cache: EntryCache) -> torch.Tensor:
+        s = self.spec
+        policy = getattr(ctx, "products", None)
+        if not cache.writes:
+            raise NotImplementedError("this mixer writes its own keys and values: it cannot borrow another entry's cache")
+        k_plane, v_plane = cache.planes["k"], cache.planes["v"]
+        qkv = ops.linear(x, self.qkv_weight, policy=policy)
+        ops.qk_rownorm_store(qkv, 0, self.q_width, self.q_width + self.k_width, self.q_width, self.k_width, self.v_width,
+                             self.q_norm, self.k_norm, s.qk_norm_eps, ctx.slots[cache.group], k_plane, v_plane)
+        out = torch.empty((x.shape[0], s.num_heads * s.value_dim), dtype=x.dtype, device=x.device)
+        run, (items, n_items) = self._runs(ctx)
+        ops.sink_attention(qkv, qkv.shape[1], out, k_plane, v_plane, ctx.block_tables[cache.group], ctx.ctx_lens, ctx.cu_q,
+                           items, n_items, run, self.r1, self.r2, self.sink, self.talk, s.num_heads, s.num_kv_heads,
+                           s.key_dim, s.value_dim, cache.block_size, s.window or 0, s.scale)
+        return ops.linear(out, self.out_weight, policy=policy)

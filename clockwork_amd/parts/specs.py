@@ -77,8 +77,127 @@ class TokenEmbeddingSpec:
 @dataclass(frozen=True)
 class LinearHeadSpec:
     """logits = rows @ W^T with W [vocab, hidden], no bias, float32 logits. ``tied``: W is the
-    embedding's table (one buffer, two uses) unless the checkpoint brings a head of its own."""
+    embedding's table (one buffer, two uses) unless the checkpoint brings a head of its own.
+    ``softcap`` c: the logits are capped, c * tanh(logits / c)."""
 
     vocab_size: int
     hidden_size: int
     tied: bool = False
+    softcap: Optional[float] = None  # logits <- softcap * tanh(logits / softcap)
+
+
+@dataclass(frozen=True)
+class LayerNormSpec:
+    """y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight + bias; statistics in float32."""
+
+    size: int
+    eps: float
+    bias: bool = True
+
+
+@dataclass(frozen=True)
+class PositionTableEmbeddingSpec:
+    """The residual stream starts as scale * table[id] + positions[p], p the token's index in its
+    request; ``max_positions`` None: no position table (a scaled lookup)."""
+
+    vocab_size: int
+    hidden_size: int
+    scale: float = 1.0
+    max_positions: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class GatedMLPSpec:
+    """down(act(gate(x)) * up(x)), no biases; ``activation`` "silu" or "gelu_tanh"
+    (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))))."""
+
+    hidden_size: int
+    intermediate_size: int
+    activation: str = "gelu_tanh"
+
+    def __post_init__(self):
+        if self.activation not in ("silu", "gelu_tanh"):
+            raise ValueError(f"activation {self.activation!r}: expected 'silu' or 'gelu_tanh'")
+
+
+@dataclass(frozen=True)
+class SinkAttentionSpec:
+    """Softmax attention with grouped query heads over a paged cache of keys [kv_heads, key_dim]
+    and values [kv_heads, value_dim], with options that plain attention has not:
+
+    * ``qk_norm``: "projection" - queries and keys are RMS-normed as whole projections (all heads
+      of a token as one vector, a weight of that size each) before they are cut into heads; None.
+    * ``distance_bias``: the score of query i and key j of head h loses r1[h] * log(1 + r2[h] * (i - j)).
+    * ``sink``: the softmax denominator of head h has the extra term exp(sink[h]): no key, no value.
+    * ``talking_heads``: the normalised weights are mixed across heads by a learned
+      [heads, heads] matrix before they are applied; head h applies its mixed weights to the
+      values of its own key/value head.
+    * ``window`` W: a token sees itself and the W - 1 tokens before it; None: all of them.
+
+    No rotation or other position encoding is applied, no biases."""
+
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    scale: float
+    window: Optional[int] = None
+    qk_norm: Optional[str] = "projection"
+    qk_norm_eps: float = 1e-6
+    distance_bias: bool = True
+    sink: bool = True
+    talking_heads: bool = True
+
+    def __post_init__(self):
+        if self.num_heads < 1 or self.num_kv_heads < 1 or self.num_heads % self.num_kv_heads:
+            raise ValueError(f"num_heads {self.num_heads} is not a multiple of num_kv_heads {self.num_kv_heads}")
+        if self.key_dim < 1 or self.value_dim < 1:
+            raise ValueError("key_dim and value_dim must be positive")
+        if self.window is not None and self.window < 1:
+            raise ValueError(f"window must be positive, got {self.window}")
+        if self.qk_norm not in (None, "projection"):
+            raise ValueError(f"qk_norm {self.qk_norm!r}: expected 'projection' or None")
+
+
+@dataclass(frozen=True)
+class DecayedLinearAttentionSpec:
+    """Linear attention with a matrix state per head and a decay per key channel:
+    S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T (q_t * key_dim^-1/2), S float32, zero at a
+    request's start. a_t = sigmoid(A2 (A1 x_t) + b)^(1/tau) with A1 [decay_rank, hidden]. Each
+    head's o_t is RMS-normed over value_dim with one weight shared by the heads, the heads are
+    concatenated, multiplied by silu(G x_t) and projected back to hidden_size."""
+
+    hidden_size: int
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    decay_rank: int
+    tau: float
+    norm_eps: float
+
+    def __post_init__(self):
+        if min(self.num_heads, self.key_dim, self.value_dim, self.decay_rank) < 1:
+            raise ValueError("heads, key_dim, value_dim and decay_rank must be positive")
+        if not self.tau > 0:
+            raise ValueError(f"tau must be positive, got {self.tau}")
+
+
+@dataclass(frozen=True)
+class PairMixerSpec:
+    """Two mixers side by side on the same input; the result is the mean of their outputs, each
+    first RMS-normed over the model width with a weight of its own."""
+
+    hidden_size: int
+    left: Any
+    right: Any
+    eps: float
+
+
+@dataclass(frozen=True)
+class BranchGateSpec:
+    """Sigmoid gates on a block's branches: branch b's output is multiplied element by element by
+    sigmoid(W_b x + c_b), x the block's normed input; ``branches`` gates of hidden_size each."""
+
+    hidden_size: int
+    branches: int = 2

@@ -28,12 +28,17 @@ class Architecture:
     parse_config: Callable[[dict], Any]
     build_spec: Callable[[Any], ModelSpec]
     weight_plan: Callable[[Any, ModelSpec], list[WeightTarget]]
+    # optional: ``sizes_from_checkpoint(config dict, {tensor name: shape}) -> config dict`` fills in
+    # sizes that the design leaves to the shapes of the checkpoint's tensors; called before
+    # ``parse_config`` when the weights come from a checkpoint
+    sizes_from_checkpoint: Any = None
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}
 _BUILTIN_ARCHITECTURES = {
     "Qwen2ForCausalLM": "clockwork_amd.models.qwen2",
     "qwen2": "clockwork_amd.models.qwen2",
+    "Fuvavik": "clockwork_amd.models.fuvavik",
 }
 
 
@@ -48,7 +53,7 @@ def unregister_architecture(names: list[str]) -> None:
 
 
 def resolve_architecture(config: dict) -> Architecture:
-    """Pick the architecture by ``architectures[0]``, else by ``model_type``.
+    """Pick the architecture by ``architectures[0]``, else by ``model_type``, else by ``architecture``.
 
     Anything unknown is refused (the reference refuses every model_type but its own,
     clockwork/engine/loader.py:70-71; an architecture's ``parse_config`` repeats that check
@@ -60,6 +65,8 @@ def resolve_architecture(config: dict) -> Architecture:
         keys.append(archs[0])
     if config.get("model_type") is not None:
         keys.append(config["model_type"])
+    if isinstance(config.get("architecture"), str):  # a configuration that names its design in one word
+        keys.append(config["architecture"])
     for key in keys:
         if key not in _ARCHITECTURES and key in _BUILTIN_ARCHITECTURES:
             importlib.import_module(_BUILTIN_ARCHITECTURES[key])
@@ -84,9 +91,17 @@ _BUILTIN_PARTS = {
     "SwiGLUSpec": ("clockwork_amd.parts.mlp", "SwiGLU"),
     "TokenEmbeddingSpec": ("clockwork_amd.parts.embedding", "TokenEmbedding"),
     "LinearHeadSpec": ("clockwork_amd.parts.embedding", "LinearHead"),
+    "PositionTableEmbeddingSpec": ("clockwork_amd.parts.embedding", "PositionTableEmbedding"),
+    "LayerNormSpec": ("clockwork_amd.parts.norm", "LayerNorm"),
+    "GatedMLPSpec": ("clockwork_amd.parts.mlp", "GatedMLP"),
+    "SinkAttentionSpec": ("clockwork_amd.parts.sink_attention", "SinkAttention"),
+    "DecayedLinearAttentionSpec": ("clockwork_amd.parts.linear_attention", "DecayedLinearAttention"),
+    "PairMixerSpec": ("clockwork_amd.parts.pair", "PairMixer"),
+    "BranchGateSpec": ("clockwork_amd.parts.block", "BranchGate"),
 }
 _ARRANGEMENTS: dict[str, Callable[..., Any]] = {}
-_BUILTIN_ARRANGEMENTS = {"prenorm": ("clockwork_amd.parts.block", "PreNormBlock")}
+_BUILTIN_ARRANGEMENTS = {"prenorm": ("clockwork_amd.parts.block", "PreNormBlock"),
+                         "parallel": ("clockwork_amd.parts.block", "ParallelBlock")}
 
 
 def register_part(spec_type: type, factory: Callable[[Any], Any]) -> None:

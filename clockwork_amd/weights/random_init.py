@@ -1,7 +1,7 @@
 """Random weights from a configuration and a seed, as checkpoint tensors or as a model folder.
 
 Distributions: matrices and embeddings N(0, 0.02), q/k/v biases N(0, 0.02), norm
-weights 1 + U(-0.1, 0.1). Each checkpoint tensor has a generator of its own,
+weights 1 + U(-0.1, 0.1); a part may also ask for U(lo, hi) or for the identity plus N(0, std). Each checkpoint tensor has a generator of its own,
 seeded from the seed and the tensor's position in the sorted list of names, so a
 tensor's values depend on neither the others nor the order of generation.
 """
@@ -57,6 +57,12 @@ class RandomSource:
         elif init[0] == "one_plus_uniform":
             t = torch.empty(shape, dtype=torch.float32, device=self.device)
             t.uniform_(-float(init[1]), float(init[1]), generator=gen).add_(1.0)
+        elif init[0] == "uniform":
+            t = torch.empty(shape, dtype=torch.float32, device=self.device)
+            t.uniform_(float(init[1]), float(init[2]), generator=gen)
+        elif init[0] == "eye_plus_normal":
+            t = torch.empty(shape, dtype=torch.float32, device=self.device)
+            t.normal_(0.0, float(init[1]), generator=gen).add_(torch.eye(shape[0], shape[1], device=self.device))
         elif init[0] == "zeros":
             t = torch.zeros(shape, dtype=torch.float32, device=self.device)
         else:
