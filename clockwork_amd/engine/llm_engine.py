@@ -70,6 +70,10 @@ class LLMEngine:
         )
         self.tokenizer = tokenizer
         self.manager = self.runner.manager
+        # a model with a position table of its own ends there, whatever the configuration allows
+        limit = self.runner.spec.max_positions
+        if limit is not None and cfg.model.max_model_len > limit:
+            cfg.set("max_model_len", limit)
         if cfg.model.tune_products:
             chunk = cfg.scheduler.max_num_batched_tokens
             if cfg.scheduler.max_prefill_chunk > 0:

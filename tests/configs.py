@@ -79,3 +79,47 @@ LAYER_32B = dict(
     num_key_value_heads=8, intermediate_size=27648, rms_norm_eps=1e-6, rope_theta=1000000.0,
     tie_word_embeddings=False,
 )
+
+
+# ---- Fuvavik: small models that differ in every size and constant; layers of one model differ too.
+def _fuvavik_layer(heads, kv_heads, dim, vdim, scale, window, r_heads, r_dim, r_vdim, tau, rank, ff):
+    return {
+        "type": "parallel",
+        "mixer": {
+            "left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "mask": {"size": window}},
+            "right": {"heads": r_heads, "dim": r_dim, "vdim": r_vdim, "tau": tau, "rank": rank},
+        },
+        "mlp": None if ff is None else {"kind": "dense", "ff": ff},
+    }
+
+
+# two layers that share nothing: grouped heads with key and value sizes apart and a window of 9
+# beside a recurrence of rank 5; then one key/value head per query head, a window of 33, no
+# feed-forward
+FUVAVIK_A = {
+    "architecture": "Fuvavik", "vocab": 300, "width": 96, "max_positions": 640,
+    "embedding": {"scale": 2.0}, "norm": {"eps": 1e-5}, "logit_softcap": 20.0,
+    "layers": [
+        _fuvavik_layer(4, 2, 24, 16, 0.2, 9, 2, 12, 20, 4.0, 5, 72),
+        _fuvavik_layer(6, 6, 16, 16, 0.25, 33, 3, 20, 8, 16.0, 3, None),
+    ],
+}
+# a width that is no multiple of 8, one key/value head for three query heads, a window longer than
+# any request of the tests (every key is seen), a single recurrent head with tau = 1, a window of 1
+FUVAVIK_B = {
+    "architecture": "Fuvavik", "vocab": 127, "width": 100, "max_positions": 700,
+    "embedding": {"scale": 0.5}, "norm": {"eps": 3e-4}, "logit_softcap": 7.5,
+    "layers": [
+        _fuvavik_layer(3, 1, 40, 24, 0.16, 300, 1, 64, 64, 1.0, 16, 50),
+        _fuvavik_layer(2, 1, 8, 32, 0.35, 1, 4, 6, 10, 2.5, 2, 130),
+        _fuvavik_layer(3, 1, 40, 24, 0.16, 300, 1, 64, 64, 1.0, 16, 50),
+    ],
+}
+# one head everywhere and sizes of 1 where the design allows them
+FUVAVIK_C = {
+    "architecture": "Fuvavik", "vocab": 64, "width": 48, "max_positions": 200,
+    "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+    "layers": [_fuvavik_layer(1, 1, 32, 8, 0.18, 17, 1, 16, 4, 8.0, 1, 24)],
+}
+# name -> (config, weight seed, cache block size)
+FUVAVIK_CONFIGS = {"FA": (FUVAVIK_A, 21, 8), "FB": (FUVAVIK_B, 22, 16), "FC": (FUVAVIK_C, 23, 4)}
