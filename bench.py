@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16] [--shape 1.5b]
     python bench.py --workload mixed|arrivals|agent [--shape 7b] [--requests 64]
+    python bench.py --design fuvavik [--size s|m|l] [--layers L] [--batch B]
 
 Default workload: the layer sizes of Qwen2.5-1.5B with random weights (seed 2), bfloat16,
 8 requests that each hold a 2048-token prompt, context limit 4096, pages of 16 tokens. A
@@ -491,6 +492,84 @@ def measure_decode_attention_grid() -> dict:
             "grid": grid}
 
 
+# Layer sizes for ``--design fuvavik``: widths, head counts and feed-forwards of the Qwen2.5
+# 0.5B / 1.5B / 7B layers, a window of half the prompt, a recurrence of as many heads with a
+# 64 x 128 state each. Beside each the Qwen2 layer of equal width, heads and feed-forward runs.
+FUVAVIK_SIZES = {
+    "s": dict(width=896, heads=14, kv_heads=2, dim=64, vdim=64, window=1024, r_heads=14, r_dim=64, r_vdim=64, rank=16,
+              ff=4864, layers=4),
+    "m": dict(width=1536, heads=12, kv_heads=2, dim=128, vdim=128, window=1024, r_heads=12, r_dim=64, r_vdim=128, rank=32,
+              ff=8960, layers=4),
+    "l": dict(width=3584, heads=28, kv_heads=4, dim=128, vdim=128, window=1024, r_heads=28, r_dim=64, r_vdim=128, rank=64,
+              ff=18944, layers=2),
+}
+DESIGN_VOCAB = 32768
+
+
+def fuvavik_config(size: dict, layers: int, max_positions: int) -> dict:
+    layer = {
+        "type": "parallel",
+        "mixer": {
+            "left": {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"],
+                     "scale": size["dim"] ** -0.5, "mask": {"size": size["window"]}},
+            "right": {"heads": size["r_heads"], "dim": size["r_dim"], "vdim": size["r_vdim"], "tau": 16.0, "rank": size["rank"]},
+        },
+        "mlp": {"kind": "dense", "ff": size["ff"]},
+    }
+    return {"architecture": "Fuvavik", "vocab": DESIGN_VOCAB, "width": size["width"], "max_positions": max_positions,
+            "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "layers": [layer] * layers}
+
+
+def qwen2_config_like(size: dict, layers: int, max_positions: int) -> dict:
+    """The closest model the engine had before: Qwen2 blocks of the same width, heads, head size,
+    feed-forward, layers and vocabulary."""
+    return dict(QWEN25_1P5B, vocab_size=DESIGN_VOCAB, hidden_size=size["width"], num_hidden_layers=layers,
+                num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
+                intermediate_size=size["ff"], max_position_embeddings=max_positions, tie_word_embeddings=True)
+
+
+def run_design(args) -> dict:
+    """Prefill (one 2048-token prompt) and decode (``--batch`` requests behind 2048-token prompts,
+    through the engine's own loop, greedy) of the design at one size, and of the Qwen2 model of
+    equal size beside it. Random weights, bfloat16 unless --dtype says otherwise."""
+    import torch
+
+    from clockwork_amd.config.engine import EngineConfig
+    from clockwork_amd.engine.model_runner import GRAPH_BATCH_SIZES, ModelRunner
+
+    size = FUVAVIK_SIZES[args.size]
+    layers = args.layers if args.layers is not None else size["layers"]
+    context = context_of(args)
+    out = {"design": args.design, "size": {**size, "layers": layers, "vocab": DESIGN_VOCAB}, "dtype": args.dtype,
+           "prompt_len": args.prompt_len, "batch": args.batch, "steps": args.steps,
+           "data": "synthetic: uniform random token ids, random weights (seed 2)"}
+    configs = {args.design: fuvavik_config(size, layers, context), "qwen2 of equal size": qwen2_config_like(size, layers, context)}
+    for name, config in configs.items():
+        cfg = EngineConfig.defaults(
+            f"random:{name}", dtype=args.dtype, max_model_len=context, block_size=BLOCK,
+            num_blocks=max(args.batch, 1) * context // BLOCK, enable_prefix_cache=False, watermark=0.0,
+            max_num_seqs=max(args.batch, 1), max_num_batched_tokens=max(PROMPT_LEN, args.batch),
+            weights="random_device", weight_seed=2,
+        )
+        runner = ModelRunner(cfg, config_dict=config)
+        if not args.no_tune:
+            runner.tune_products([PROMPT_LEN, *[b for b in GRAPH_BATCH_SIZES if b <= args.batch]])
+        t = time_prefill(cfg, runner, total=args.prompt_len)
+        elapsed, _ = time_decode(cfg, runner, args.batch, args.steps, args.warmup, None, args.prompt_len)
+        out[name] = {
+            "prefill_tokens_per_s": round(args.prompt_len / t, 1), "prefill_ms": round(1e3 * t, 3),
+            "decode_tokens_per_s": round(args.batch * args.steps / elapsed, 1),
+            "decode_ms_per_step": round(1e3 * elapsed / args.steps, 4),
+            "weight_bytes_per_step": runner.model.weight_bytes_per_step(),
+        }
+        del runner
+        torch.cuda.empty_cache()
+    a, b = out[args.design], out["qwen2 of equal size"]
+    out["ratio_to_qwen2"] = {"prefill": round(a["prefill_tokens_per_s"] / b["prefill_tokens_per_s"], 3),
+                             "decode": round(a["decode_tokens_per_s"] / b["decode_tokens_per_s"], 3)}
+    return out
+
+
 def prefill_flops(spec, model, T: int) -> float:
     """2 * T * (matrix parameters of the layers) + causal attention + one row of the output head."""
     layer_params = 0
@@ -528,6 +607,9 @@ def main() -> int:
     ap.add_argument("--peaks", action="store_true", help="measure a device copy and a large library product instead")
     ap.add_argument("--decode-attention-grid", action="store_true",
                     help="time the attention part alone over the reference's grid of batch sizes and context lengths instead")
+    ap.add_argument("--design", default=None, choices=("fuvavik",),
+                    help="measure another design's prefill and decode beside the Qwen2 model of equal size instead")
+    ap.add_argument("--size", default="m", choices=sorted(FUVAVIK_SIZES), help="--design: which layer sizes")
     ap.add_argument("--temperature", type=float, default=0.0, help="sample instead of the greedy decoding of the recorded benchmark")
     ap.add_argument("--top-k", type=int, default=-1)
     ap.add_argument("--top-p", type=float, default=1.0)
@@ -543,6 +625,9 @@ def main() -> int:
         return 0
     if args.decode_attention_grid:
         print(json.dumps(measure_decode_attention_grid()))
+        return 0
+    if args.design is not None:
+        print(json.dumps(run_design(args)))
         return 0
     if args.workload == "agent":
         print(json.dumps(run_agent(args)))
