@@ -183,3 +183,250 @@ CW_EXPORT int cw_linear_recurrence(int dtype, const void* proj, int64_t stride, 
 #undef CW_LAUNCH
   return cw_launch_status();
 }
+
+// ======================================================================================
+// The same recurrence for long portions, cut into segments of tokens that run side by side.
+//
+//   prepare:   per token and key channel the decay a (float32, through log-sigmoid), the scaled
+//              query and the key as float32 rows [T, heads * dim]: the walks below read them
+//              with addresses that do not depend on the lane, so they arrive in scalar registers.
+//   segments:  every (segment, head) walks its tokens from a zero state: what the segment adds to
+//              the state (float32 [dim, vdim]) and the product of its decays per channel.
+//   carry:     per request and head, segment after segment: start(s + 1) = decay(s) * start(s) +
+//              added(s), from the request's state slot; the last one is the slot's new state.
+//   outputs:   every (segment, head) walks its tokens again from its start state: o_t = S_t^T q_t.
+//   finish:    RMS norm over vdim, weight, silu(gate), cast: one wave per (token, head).
+//
+// In the walks a thread owns one column of the state with all its rows in registers (dim <= 128),
+// a wave 64 columns; nothing is exchanged between threads. The sums are the same as in the
+// token-by-token kernel but for the place of the parentheses: S_t = A S_start + (local sum).
+// ======================================================================================
+#define LRS_MAX_DIM 128
+
+struct SegParams {
+  const void* proj;
+  int64_t stride;
+  int q_off, k_off, v_off, g_off, u_off;
+  const void* a2;
+  const float* a2b;
+  const float* norm_w;
+  float* state;
+  const int* state_slots;
+  const int* cu_q;
+  const int* seg_items;   // [n_segments, 4]: request, first token of the segment (in the portion), tokens, index of the segment in its request
+  const int* req_first;   // [R + 1]: first segment of each request in seg_items
+  float* dec;             // [T, heads * dim] decays
+  float* qf;              // [T, heads * dim]
+  float* kf;              // [T, heads * dim]
+  float* added;           // [n_segments, heads, dim, vdim]
+  float* seg_decay;       // [n_segments, heads, dim]
+  float* raw;             // [T, heads * vdim] outputs before norm and gate
+  void* out;
+  int heads, dim, vdim, rank, n_slots, n_tokens;
+  float q_scale, inv_tau, eps;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void lrs_prepare_kernel(SegParams p) {
+  const int HD = p.heads * p.dim;
+  const int64_t n = (int64_t)p.n_tokens * HD;
+  const T* proj = (const T*)p.proj;
+  const T* a2 = (const T*)p.a2;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * 256) {
+    const int64_t t = idx / HD;
+    const int c = (int)(idx - t * HD);
+    const T* row = proj + t * p.stride;
+    float z = p.a2b ? p.a2b[c] : 0.0f;
+    const T* w = a2 + (int64_t)c * p.rank;
+    for (int e = 0; e < p.rank; ++e) z += cw_to_float(w[e]) * cw_to_float(row[p.u_off + e]);
+    const float ls = z < 0.0f ? z - log1pf(expf(z)) : -log1pf(expf(-z));
+    p.dec[idx] = expf(ls * p.inv_tau);
+    p.qf[idx] = cw_to_float(row[p.q_off + c]) * p.q_scale;
+    p.kf[idx] = cw_to_float(row[p.k_off + c]);
+  }
+}
+
+// MODE 0: from zero, leaves ``added`` and ``seg_decay``; MODE 1: from the start state in ``added``
+// (the carry kernel has turned it into that), writes the raw outputs.
+template <typename T, int DIM, int MODE>
+__global__ __launch_bounds__(64) void lrs_walk_kernel(SegParams p) {
+  const int seg = blockIdx.x, h = blockIdx.y;
+  const int v = blockIdx.z * 64 + threadIdx.x;
+  const int r = p.seg_items[4 * seg], tok0 = p.seg_items[4 * seg + 1], ntok = p.seg_items[4 * seg + 2];
+  const int q_len = p.cu_q[r + 1] - p.cu_q[r];
+  const int slot = p.state_slots[r];
+  if (tok0 >= q_len || slot < 0 || slot >= p.n_slots) return;
+  const int nt = min(ntok, q_len - tok0);
+  const int64_t row0 = p.cu_q[r] + tok0;
+  const int D = p.dim, V = p.vdim, HD = p.heads * p.dim;
+  const bool live = v < V;
+  const int vc = live ? v : V - 1;
+  float S[DIM];
+  float* mine = p.added + (((int64_t)seg * p.heads + h) * D) * V;
+  if (MODE == 1) {
+#pragma unroll
+    for (int d = 0; d < DIM; ++d) S[d] = d < D ? mine[(int64_t)d * V + vc] : 0.0f;
+  } else {
+#pragma unroll
+    for (int d = 0; d < DIM; ++d) S[d] = 0.0f;
+  }
+  float A[MODE == 0 ? DIM : 1];
+  if (MODE == 0) {
+#pragma unroll
+    for (int d = 0; d < DIM; ++d) A[d] = 1.0f;
+  }
+  const T* proj = (const T*)p.proj;
+  for (int t = 0; t < nt; ++t) {
+    const int64_t row = row0 + t;
+    // the same addresses in every lane: scalar loads
+    const float* a = p.dec + row * HD + h * D;
+    const float* k = p.kf + row * HD + h * D;
+    const float* q = p.qf + row * HD + h * D;
+    const float vv = cw_to_float(proj[row * p.stride + p.v_off + h * V + vc]);
+    float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
+#pragma unroll
+    for (int d = 0; d < DIM; d += 4) {
+      if (d < D) {  // D is a multiple of 4 here (the host sees to it)
+        S[d] = a[d] * S[d] + k[d] * vv;
+        S[d + 1] = a[d + 1] * S[d + 1] + k[d + 1] * vv;
+        S[d + 2] = a[d + 2] * S[d + 2] + k[d + 2] * vv;
+        S[d + 3] = a[d + 3] * S[d + 3] + k[d + 3] * vv;
+        if (MODE == 1) {
+          o0 += q[d] * S[d];
+          o1 += q[d + 1] * S[d + 1];
+          o2 += q[d + 2] * S[d + 2];
+          o3 += q[d + 3] * S[d + 3];
+        } else if (threadIdx.x == 0 && blockIdx.z == 0) {
+          A[d] *= a[d]; A[d + 1] *= a[d + 1]; A[d + 2] *= a[d + 2]; A[d + 3] *= a[d + 3];
+        }
+      }
+    }
+    if (MODE == 1 && live) p.raw[row * (int64_t)(p.heads * V) + h * V + v] = (o0 + o1) + (o2 + o3);
+  }
+  if (MODE == 0) {
+    if (live) {
+#pragma unroll
+      for (int d = 0; d < DIM; ++d)
+        if (d < D) mine[(int64_t)d * V + v] = S[d];
+    }
+    if (threadIdx.x == 0 && blockIdx.z == 0) {
+      float* sd = p.seg_decay + ((int64_t)seg * p.heads + h) * D;
+#pragma unroll
+      for (int d = 0; d < DIM; ++d)
+        if (d < D) sd[d] = A[d];
+    }
+  }
+}
+
+// per (request, head, 256 state elements): walk the request's segments in order
+__global__ __launch_bounds__(256) void lrs_carry_kernel(SegParams p) {
+  const int r = blockIdx.x, h = blockIdx.y;
+  const int64_t e = (int64_t)blockIdx.z * 256 + threadIdx.x;  // element d * V + v
+  const int D = p.dim, V = p.vdim;
+  const int slot = p.state_slots[r];
+  const int q_len = p.cu_q[r + 1] - p.cu_q[r];
+  if (e >= (int64_t)D * V || slot < 0 || slot >= p.n_slots || q_len <= 0) return;
+  const int d = (int)(e / V);
+  float* st = p.state + (((int64_t)slot * p.heads + h) * D) * V + e;
+  float S = *st;
+  for (int seg = p.req_first[r]; seg < p.req_first[r + 1]; ++seg) {
+    if (p.seg_items[4 * seg + 1] >= q_len) break;  // segments past the request's tokens (a batch of fixed shape)
+    float* mine = p.added + (((int64_t)seg * p.heads + h) * D) * V + e;
+    const float add = *mine;
+    *mine = S;  // the segment's start state, for the second walk
+    S = p.seg_decay[((int64_t)seg * p.heads + h) * D + d] * S + add;
+  }
+  *st = S;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void lrs_finish_kernel(SegParams p) {
+  const int V = p.vdim, Hn = p.heads;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t item = (int64_t)blockIdx.x * 4 + wave;  // (token, head)
+  if (item >= (int64_t)p.n_tokens * Hn) return;
+  const int64_t t = item / Hn;
+  const int h = (int)(item - t * Hn);
+  const float* o = p.raw + t * (int64_t)(Hn * V) + h * V;
+  float ss = 0.0f;
+  for (int c = lane; c < V; c += 64) ss += o[c] * o[c];
+  float inv = 1.0f;
+  if (p.norm_w) inv = 1.0f / sqrtf(cw_wave_sum(ss) / (float)V + p.eps);
+  const T* proj = (const T*)p.proj;
+  T* out = (T*)p.out;
+  for (int c = lane; c < V; c += 64) {
+    float val = o[c] * inv;
+    if (p.norm_w) val *= p.norm_w[c];
+    if (p.g_off >= 0) {
+      const float g = cw_to_float(proj[t * p.stride + p.g_off + h * V + c]);
+      val *= g / (1.0f + expf(-g));
+    }
+    out[t * (int64_t)(Hn * V) + h * V + c] = cw_from_float<T>(val);
+  }
+}
+
+// dim a multiple of 4 up to 128
+CW_EXPORT int cw_linear_recurrence_segments_supported(int dim, int vdim) {
+  return dim > 0 && dim <= LRS_MAX_DIM && dim % 4 == 0 && vdim > 0 ? 1 : 0;
+}
+
+// floats of workspace: dec, qf, kf [T, heads * dim] each, added [segments, heads, dim, vdim],
+// seg_decay [segments, heads, dim], raw [T, heads * vdim]
+CW_EXPORT int64_t cw_linear_recurrence_segments_workspace_floats(int n_tokens, int n_segments, int heads, int dim, int vdim) {
+  return 3 * (int64_t)n_tokens * heads * dim + (int64_t)n_segments * heads * dim * (vdim + 1) + (int64_t)n_tokens * heads * vdim;
+}
+
+CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t stride, int q_off, int k_off, int v_off,
+                                            int g_off, int u_off, const void* a2, const float* a2b, const float* norm_w,
+                                            float* state, int n_slots, const int* state_slots, const int* cu_q,
+                                            const int* seg_items, int n_segments, const int* req_first, float* workspace,
+                                            void* out, int n_requests, int n_tokens, int heads, int dim, int vdim, int rank,
+                                            float q_scale, float inv_tau, float eps, hipStream_t stream) {
+  if (n_requests < 0 || n_tokens < 0 || n_segments < 0 || !proj || !a2 || !state || !state_slots || !cu_q || !seg_items ||
+      !req_first || !workspace || !out)
+    return CW_ERR_ARG;
+  if (heads <= 0 || rank <= 0 || n_slots <= 0 || q_off < 0 || k_off < 0 || v_off < 0 || u_off < 0) return CW_ERR_ARG;
+  if (q_off + heads * dim > stride || k_off + heads * dim > stride || v_off + heads * vdim > stride ||
+      u_off + rank > stride || (g_off >= 0 && g_off + heads * vdim > stride))
+    return CW_ERR_ARG;
+  if (!cw_linear_recurrence_segments_supported(dim, vdim)) return CW_ERR_SIZE;
+  if (heads > 65535 || (vdim + 63) / 64 > 65535) return CW_ERR_SIZE;
+  if (n_requests == 0 || n_tokens == 0 || n_segments == 0) return CW_OK;
+  SegParams p;
+  p.proj = proj; p.stride = stride; p.q_off = q_off; p.k_off = k_off; p.v_off = v_off; p.g_off = g_off; p.u_off = u_off;
+  p.a2 = a2; p.a2b = a2b; p.norm_w = norm_w; p.state = state; p.state_slots = state_slots; p.cu_q = cu_q;
+  p.seg_items = seg_items; p.req_first = req_first; p.out = out;
+  p.heads = heads; p.dim = dim; p.vdim = vdim; p.rank = rank; p.n_slots = n_slots; p.n_tokens = n_tokens;
+  p.q_scale = q_scale; p.inv_tau = inv_tau; p.eps = eps;
+  const int64_t THD = (int64_t)n_tokens * heads * dim;
+  p.dec = workspace; p.qf = p.dec + THD; p.kf = p.qf + THD;
+  p.added = p.kf + THD;
+  p.seg_decay = p.added + (int64_t)n_segments * heads * dim * vdim;
+  p.raw = p.seg_decay + (int64_t)n_segments * heads * dim;
+  int64_t pb = (THD + 255) / 256;
+  if (pb > 65536) pb = 65536;
+  const dim3 walk_grid(n_segments, heads, (vdim + 63) / 64);
+  const dim3 carry_grid(n_requests, heads, (unsigned)(((int64_t)dim * vdim + 255) / 256));
+  const unsigned finish_blocks = (unsigned)(((int64_t)n_tokens * heads + 3) / 4);
+#define CW_WALK(T_, DIM_)                                                                          \
+  do {                                                                                             \
+    hipLaunchKernelGGL((lrs_walk_kernel<T_, DIM_, 0>), walk_grid, dim3(64), 0, stream, p);         \
+    hipLaunchKernelGGL(lrs_carry_kernel, carry_grid, dim3(256), 0, stream, p);                     \
+    hipLaunchKernelGGL((lrs_walk_kernel<T_, DIM_, 1>), walk_grid, dim3(64), 0, stream, p);         \
+  } while (0)
+#define CW_ALL(T_)                                                                                 \
+  do {                                                                                             \
+    hipLaunchKernelGGL((lrs_prepare_kernel<T_>), dim3((unsigned)pb), dim3(256), 0, stream, p);     \
+    if (dim <= 16) CW_WALK(T_, 16);                                                                \
+    else if (dim <= 32) CW_WALK(T_, 32);                                                           \
+    else if (dim <= 64) CW_WALK(T_, 64);                                                           \
+    else CW_WALK(T_, 128);                                                                         \
+    hipLaunchKernelGGL((lrs_finish_kernel<T_>), dim3(finish_blocks), dim3(256), 0, stream, p);     \
+  } while (0)
+  if (dtype == CW_F32) CW_ALL(float);
+  else if (dtype == CW_BF16) CW_ALL(bf16_t);
+  else return CW_ERR_DTYPE;
+#undef CW_ALL
+#undef CW_WALK
+  return cw_launch_status();
+}

@@ -134,6 +134,10 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
         "linear_recurrence": {
             "cw_linear_recurrence_supported": [I, I],
             "cw_linear_recurrence": [I, P, L, I, I, I, I, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, F, F, P],
+            "cw_linear_recurrence_segments_supported": [I, I],
+            "cw_linear_recurrence_segments_workspace_floats": [I, I, I, I, I],
+            "cw_linear_recurrence_segments": [I, P, L, I, I, I, I, I, P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, I, I,
+                                              F, F, F, P],
         },
         "sampling": {
             "cw_argmax_chunks": [I],
@@ -1421,4 +1425,39 @@ def linear_recurrence(proj, q_off: int, k_off: int, v_off: int, g_off: int, u_of
         dtype_code(proj.dtype), _ptr(proj), width, q_off, k_off, v_off, g_off, u_off, _ptr(a2), _ptr(a2_bias),
         _ptr(norm_weight), _ptr(state), state.shape[0], _ptr(state_slots), _ptr(cu_q), _ptr(out), n_requests, heads, dim,
         vdim, a2.shape[1], float(q_scale), 1.0 / float(tau), float(eps), _stream()), "linear_recurrence")
+    return out
+
+
+def linear_recurrence_segments_supported(dim: int, vdim: int) -> bool:
+    return bool(_load("linear_recurrence").cw_linear_recurrence_segments_supported(dim, vdim))
+
+
+def linear_recurrence_segments(proj, q_off: int, k_off: int, v_off: int, g_off: int, u_off: int, a2, a2_bias, norm_weight,
+                               state, state_slots, cu_q, seg_items, n_segments: int, req_first, n_requests: int, heads: int,
+                               dim: int, vdim: int, q_scale: float, tau: float, eps: float) -> torch.Tensor:
+    """``linear_recurrence`` for steps with long portions: the tokens are cut into segments that
+    are walked side by side (each from a zero state, then the segments' start states are carried
+    from the request's slot, then each is walked again for its outputs). ``seg_items`` int32
+    [n_segments, 4]: (request, first token of the segment in the request's portion, tokens, 0),
+    a request's segments in order and together; ``req_first`` int32 [R + 1]: where each
+    request's segments begin. The same arguments and result otherwise."""
+    _gpu(proj, a2, a2_bias, norm_weight, state, state_slots, cu_q, seg_items, req_first)
+    T, width = proj.shape
+    _need(a2.dim() == 2 and a2.shape[0] == heads * dim and a2.dtype == proj.dtype, "a2 must be [heads * dim, rank] in the activation type")
+    _need(a2_bias is None or (a2_bias.dtype == torch.float32 and a2_bias.numel() == heads * dim), "the decay bias must be float32 [heads * dim]")
+    _need(norm_weight is None or (norm_weight.dtype == torch.float32 and norm_weight.numel() == vdim), "the norm weight must be float32 [vdim]")
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, dim, vdim), "the state must be float32 [slots, heads, dim, vdim]")
+    _i32(state_slots, n_requests, "state_slots")
+    _i32(cu_q, n_requests + 1, "cu_q")
+    _i32(seg_items, 4 * n_segments, "seg_items")
+    _i32(req_first, n_requests + 1, "req_first")
+    lib = _load("linear_recurrence")
+    need = lib.cw_linear_recurrence_segments_workspace_floats(T, n_segments, heads, dim, vdim)
+    workspace = torch.empty(max(int(need), 1), dtype=torch.float32, device=proj.device)
+    out = torch.empty((T, heads * vdim), dtype=proj.dtype, device=proj.device)
+    _check(lib.cw_linear_recurrence_segments(
+        dtype_code(proj.dtype), _ptr(proj), width, q_off, k_off, v_off, g_off, u_off, _ptr(a2), _ptr(a2_bias),
+        _ptr(norm_weight), _ptr(state), state.shape[0], _ptr(state_slots), _ptr(cu_q), _ptr(seg_items), n_segments,
+        _ptr(req_first), _ptr(workspace), _ptr(out), n_requests, T, heads, dim, vdim, a2.shape[1], float(q_scale),
+        1.0 / float(tau), float(eps), _stream()), "linear_recurrence_segments")
     return out
