@@ -256,3 +256,313 @@ CW_EXPORT int cw_sink_attention(int dtype, const void* q, int64_t q_stride, void
 #undef CW_LAUNCH
   return cw_launch_status();
 }
+
+// ======================================================================================
+// Single tokens (one query a request): three small kernels that share a request's keys among
+// workgroups, since a request alone would leave all but one compute unit idle.
+//
+//   scores:  a workgroup per (request, run of ``sk`` keys): a thread takes one key of one
+//            key/value head, reads its row once in 16-byte pieces and multiplies it with all query
+//            heads of the group (the queries wait in LDS); scale, distance bias, mask. The scores
+//            go to a float32 workspace, each head's maximum and sum of exponentials over the run
+//            beside them.
+//   values:  the same grid: every workgroup puts the runs' maxima and sums (and the sink)
+//            together, so it knows each head's final denominator, normalises its run's scores,
+//            mixes them across heads in LDS and multiplies with its run's values: a thread takes
+//            one value column of one key/value head for all query heads of the group.
+//   merge:   the runs' partial outputs are added in order.
+// ======================================================================================
+#define SD_MAX_SK 128
+#define SD_HG 16      // query heads of a group that a thread handles at a time
+
+struct SinkDecodeParams {
+  const void* q;
+  int64_t q_stride;
+  void* out;
+  const void* k_cache;
+  const void* v_cache;
+  const int* block_tables;
+  int table_width;
+  const int* ctx_lens;
+  const int* cu_q;
+  const float* r1;
+  const float* r2;
+  const float* sink;
+  const float* talk;
+  float* scores;   // [R, heads, n_runs * sk]
+  float* stats;    // [R, n_runs, heads, 2]
+  float* partial;  // [R, n_runs, heads * vdim]
+  int heads, kv_heads, dim, vdim, block_size, window, sk, n_runs;
+  float scale;
+  int64_t cache_rows;
+};
+
+// keys that request r's single token sees: [lo, pos]; false if the request has another number of tokens
+__device__ __forceinline__ bool sd_range(const SinkDecodeParams& p, int r, int& lo, int& pos) {
+  if (p.cu_q[r + 1] - p.cu_q[r] != 1) return false;
+  pos = p.ctx_lens[r] - 1;
+  lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  return pos >= 0;
+}
+
+template <typename T> struct RowVec;
+template <> struct RowVec<float> {
+  static constexpr int N = 4;
+  __device__ static void load(const float* p, float* o) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+  }
+};
+template <> struct RowVec<bf16_t> {
+  static constexpr int N = 8;
+  __device__ static void load(const bf16_t* p, float* o) {
+    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(w[i] << 16); o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void sink_decode_scores_kernel(SinkDecodeParams p) {
+  extern __shared__ __align__(16) float smem[];
+  const int H = p.heads, G = p.kv_heads, D = p.dim, Hg = H / G, SK = p.sk;
+  const int r = blockIdx.x, run = blockIdx.y, tid = threadIdx.x;
+  int lo, pos;
+  if (!sd_range(p, r, lo, pos)) return;
+  const int k0 = lo + run * SK;
+  if (k0 > pos) return;
+  float* qs = smem;            // [H * D]
+  float* sc = qs + H * D;      // [H][SK]
+  const T* q = (const T*)p.q + (int64_t)p.cu_q[r] * p.q_stride;
+  for (int i = tid; i < H * D; i += 256) qs[i] = cw_to_float(q[i]);
+  __syncthreads();
+  const int* table = p.block_tables + (int64_t)r * p.table_width;
+  const T* kc = (const T*)p.k_cache;
+  constexpr int N = RowVec<T>::N;
+  const bool vec = D % N == 0 && !((uintptr_t)kc & 15);
+  for (int idx = tid; idx < SK * G; idx += 256) {
+    const int c = idx / SK, jj = idx - c * SK;
+    const int j = k0 + jj;
+    const bool seen = j <= pos;
+    const T* krow = kc;
+    bool there = false;
+    if (seen) {
+      const int page = table[j / p.block_size];
+      const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
+      there = page >= 0 && row < p.cache_rows;
+      if (there) krow = kc + (row * G + c) * D;
+    }
+    for (int h0 = 0; h0 < Hg; h0 += SD_HG) {
+      float acc[SD_HG];
+#pragma unroll
+      for (int e = 0; e < SD_HG; ++e) acc[e] = 0.0f;
+      if (there) {
+        if (vec) {
+          for (int d = 0; d < D; d += N) {
+            float kv[N];
+            RowVec<T>::load(krow + d, kv);
+#pragma unroll
+            for (int e = 0; e < SD_HG; ++e) {
+              if (h0 + e < Hg) {
+                const float* qv = qs + (c * Hg + h0 + e) * D + d;
+#pragma unroll
+                for (int u = 0; u < N; ++u) acc[e] += qv[u] * kv[u];
+              }
+            }
+          }
+        } else {
+          for (int d = 0; d < D; ++d) {
+            const float kv = cw_to_float(krow[d]);
+#pragma unroll
+            for (int e = 0; e < SD_HG; ++e)
+              if (h0 + e < Hg) acc[e] += qs[(c * Hg + h0 + e) * D + d] * kv;
+          }
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < SD_HG; ++e) {
+        if (h0 + e < Hg) {
+          const int g = c * Hg + h0 + e;
+          float s = acc[e] * p.scale;
+          if (p.r1) s -= p.r1[g] * log1pf(p.r2[g] * (float)max(pos - j, 0));
+          sc[g * SK + jj] = seen ? s : -INFINITY;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  const int wave = tid >> 6, lane = tid & 63;
+  float* ws = p.scores + ((int64_t)r * H) * (p.n_runs * SK) + run * SK;
+  for (int g = wave; g < H; g += 4) {
+    float m = -INFINITY;
+    for (int jj = lane; jj < SK; jj += 64) {
+      const float s = sc[g * SK + jj];
+      ws[(int64_t)g * (p.n_runs * SK) + jj] = s;
+      m = fmaxf(m, s);
+    }
+    m = cw_wave_max(m);
+    float l = 0.0f;
+    for (int jj = lane; jj < SK; jj += 64) l += expf(sc[g * SK + jj] - m);
+    l = cw_wave_sum(l);
+    if (lane == 0) {
+      float* st = p.stats + (((int64_t)r * p.n_runs + run) * H + g) * 2;
+      st[0] = m;
+      st[1] = l;
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void sink_decode_values_kernel(SinkDecodeParams p) {
+  extern __shared__ __align__(16) float smem[];
+  const int H = p.heads, G = p.kv_heads, V = p.vdim, Hg = H / G, SK = p.sk;
+  const int r = blockIdx.x, run = blockIdx.y, tid = threadIdx.x;
+  int lo, pos;
+  if (!sd_range(p, r, lo, pos)) return;
+  const int k0 = lo + run * SK;
+  if (k0 > pos) return;
+  const int runs = (pos - lo) / SK + 1;  // the runs that hold keys of this request
+  float* Pn = smem;              // [H][SK] normalised weights
+  float* Pm = Pn + H * SK;       // [H][SK] mixed
+  float* mg = Pm + H * SK;       // [H] maxima
+  float* il = mg + H;            // [H] 1 / denominators
+  int* rows = (int*)(il + H);    // [SK] cache rows of the run's keys (-1: none)
+  for (int g = tid; g < H; g += 256) {
+    float m = p.sink ? p.sink[g] : -INFINITY;
+    const float* st = p.stats + ((int64_t)r * p.n_runs * H + g) * 2;
+    for (int s = 0; s < runs; ++s) m = fmaxf(m, st[(int64_t)s * H * 2]);
+    float l = p.sink ? expf(p.sink[g] - m) : 0.0f;
+    for (int s = 0; s < runs; ++s) l += st[(int64_t)s * H * 2 + 1] * expf(st[(int64_t)s * H * 2] - m);
+    mg[g] = m;
+    il[g] = l > 0.0f ? 1.0f / l : 0.0f;
+  }
+  const int* table = p.block_tables + (int64_t)r * p.table_width;
+  for (int jj = tid; jj < SK; jj += 256) {
+    const int j = k0 + jj;
+    int row = -1;
+    if (j <= pos) {
+      const int page = table[j / p.block_size];
+      const int64_t at = (int64_t)page * p.block_size + j % p.block_size;
+      if (page >= 0 && at < p.cache_rows) row = (int)at;
+    }
+    rows[jj] = row;
+  }
+  __syncthreads();
+  const float* ws = p.scores + ((int64_t)r * H) * (p.n_runs * SK) + run * SK;
+  for (int idx = tid; idx < H * SK; idx += 256) {
+    const int g = idx / SK, jj = idx - g * SK;
+    Pn[idx] = expf(ws[(int64_t)g * (p.n_runs * SK) + jj] - mg[g]) * il[g];
+  }
+  __syncthreads();
+  const float* W = Pn;
+  if (p.talk) {
+    for (int idx = tid; idx < H * SK; idx += 256) {
+      const int h = idx / SK, jj = idx - h * SK;
+      float v = 0.0f;
+      for (int g = 0; g < H; ++g) v += p.talk[h * H + g] * Pn[g * SK + jj];
+      Pm[idx] = v;
+    }
+    __syncthreads();
+    W = Pm;
+  }
+  const int nk = min(SK, pos - k0 + 1);
+  const T* vc = (const T*)p.v_cache;
+  float* part = p.partial + ((int64_t)r * p.n_runs + run) * (H * V);
+  for (int idx = tid; idx < G * V; idx += 256) {
+    const int c = idx / V, dv = idx - c * V;
+    for (int h0 = 0; h0 < Hg; h0 += SD_HG) {
+      float acc[SD_HG];
+#pragma unroll
+      for (int e = 0; e < SD_HG; ++e) acc[e] = 0.0f;
+#pragma unroll 4
+      for (int jj = 0; jj < nk; ++jj) {
+        const int row = rows[jj];
+        const float v = row >= 0 ? cw_to_float(vc[((int64_t)row * G + c) * V + dv]) : 0.0f;
+#pragma unroll
+        for (int e = 0; e < SD_HG; ++e)
+          if (h0 + e < Hg) acc[e] += W[(c * Hg + h0 + e) * SK + jj] * v;
+      }
+#pragma unroll
+      for (int e = 0; e < SD_HG; ++e)
+        if (h0 + e < Hg) part[(c * Hg + h0 + e) * V + dv] = acc[e];
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void sink_decode_merge_kernel(SinkDecodeParams p) {
+  const int r = blockIdx.x;
+  int lo, pos;
+  if (!sd_range(p, r, lo, pos)) return;
+  const int runs = (pos - lo) / p.sk + 1;
+  const int n = p.heads * p.vdim;
+  T* out = (T*)p.out + (int64_t)p.cu_q[r] * n;
+  const float* part = p.partial + (int64_t)r * p.n_runs * n;
+  for (int i = blockIdx.y * 256 + threadIdx.x; i < n; i += gridDim.y * 256) {
+    float v = part[i];
+    for (int s = 1; s < runs; ++s) v += part[(int64_t)s * n + i];
+    out[i] = cw_from_float<T>(v);
+  }
+}
+
+// floats of workspace for R single tokens whose keys are cut into n_runs runs of sk keys
+CW_EXPORT int64_t cw_sink_decode_workspace_floats(int n_requests, int n_runs, int sk, int heads, int vdim) {
+  return (int64_t)n_requests * heads * n_runs * sk + (int64_t)n_requests * n_runs * heads * 2 +
+         (int64_t)n_requests * n_runs * heads * vdim;
+}
+
+CW_EXPORT int cw_sink_decode_supported(int heads, int kv_heads, int dim, int vdim) {
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return 0;
+  const int64_t a = ((int64_t)heads * dim + (int64_t)heads * SD_MAX_SK) * 4;
+  const int64_t b = (2 * (int64_t)heads * SD_MAX_SK + 2 * heads + SD_MAX_SK) * 4;
+  return a <= 150 * 1024 && b <= 150 * 1024 ? 1 : 0;
+}
+
+// Every request of the step has one token (requests with another count are left alone). The keys a
+// token sees ([max(0, pos - window + 1), pos]) are cut into runs of sk keys from their first;
+// n_runs is the most runs any request has (the host knows the longest context).
+CW_EXPORT int cw_sink_decode(int dtype, const void* q, int64_t q_stride, void* out, const void* k_cache,
+                             const void* v_cache, int64_t cache_rows, const int* block_tables, int table_width,
+                             const int* ctx_lens, const int* cu_q, int n_requests, int sk, int n_runs, float* workspace,
+                             const float* r1, const float* r2, const float* sink, const float* talk, int heads,
+                             int kv_heads, int dim, int vdim, int block_size, int window, float scale, hipStream_t stream) {
+  if (n_requests < 0 || !q || !out || !k_cache || !v_cache || !block_tables || !ctx_lens || !cu_q || !workspace)
+    return CW_ERR_ARG;
+  if (block_size <= 0 || table_width <= 0 || window < 0 || (r1 && !r2) || sk < 1 || sk > SD_MAX_SK || n_runs < 1)
+    return CW_ERR_ARG;
+  if (!cw_sink_decode_supported(heads, kv_heads, dim, vdim)) return CW_ERR_SIZE;
+  if (n_runs > 65535) return CW_ERR_SIZE;
+  if (n_requests == 0) return CW_OK;
+  SinkDecodeParams p;
+  p.q = q; p.q_stride = q_stride; p.out = out; p.k_cache = k_cache; p.v_cache = v_cache;
+  p.block_tables = block_tables; p.table_width = table_width; p.ctx_lens = ctx_lens; p.cu_q = cu_q;
+  p.r1 = r1; p.r2 = r2; p.sink = sink; p.talk = talk;
+  p.scores = workspace;
+  p.stats = p.scores + (int64_t)n_requests * heads * n_runs * sk;
+  p.partial = p.stats + (int64_t)n_requests * n_runs * heads * 2;
+  p.heads = heads; p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.block_size = block_size; p.window = window;
+  p.sk = sk; p.n_runs = n_runs; p.scale = scale; p.cache_rows = cache_rows;
+  const size_t smem1 = ((size_t)heads * dim + (size_t)heads * sk) * sizeof(float);
+  const size_t smem2 = (2 * (size_t)heads * sk + 2 * heads + sk) * sizeof(float);
+  const dim3 grid(n_requests, n_runs), block(256);
+  int my = (heads * vdim + 255) / 256;
+  if (my > 64) my = 64;
+#define CW_LAUNCH(T_)                                                                                                  \
+  do {                                                                                                                 \
+    if (smem1 > 48 * 1024 && hipFuncSetAttribute((const void*)sink_decode_scores_kernel<T_>,                           \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess)  \
+      return CW_ERR_LAUNCH;                                                                                            \
+    if (smem2 > 48 * 1024 && hipFuncSetAttribute((const void*)sink_decode_values_kernel<T_>,                           \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem2) != hipSuccess)  \
+      return CW_ERR_LAUNCH;                                                                                            \
+    hipLaunchKernelGGL((sink_decode_scores_kernel<T_>), grid, block, smem1, stream, p);                                \
+    hipLaunchKernelGGL((sink_decode_values_kernel<T_>), grid, block, smem2, stream, p);                                \
+    hipLaunchKernelGGL((sink_decode_merge_kernel<T_>), dim3(n_requests, my), block, 0, stream, p);                     \
+  } while (0)
+  if (dtype == CW_F32) CW_LAUNCH(float);
+  else if (dtype == CW_BF16) CW_LAUNCH(bf16_t);
+  else return CW_ERR_DTYPE;
+#undef CW_LAUNCH
+  return cw_launch_status();
+}

@@ -130,6 +130,9 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
         "sink_attention": {
             "cw_sink_attention_max_bq": [I, I, I, I],
             "cw_sink_attention": [I, P, L, P, P, P, L, P, I, P, P, P, I, I, P, P, P, P, I, I, I, I, I, I, F, P],
+            "cw_sink_decode_workspace_floats": [I, I, I, I, I],
+            "cw_sink_decode_supported": [I, I, I, I],
+            "cw_sink_decode": [I, P, L, P, P, P, L, P, I, P, P, I, I, I, P, P, P, P, P, I, I, I, I, I, I, F, P],
         },
         "linear_recurrence": {
             "cw_linear_recurrence_supported": [I, I],
@@ -1461,3 +1464,42 @@ def linear_recurrence_segments(proj, q_off: int, k_off: int, v_off: int, g_off: 
         _ptr(req_first), _ptr(workspace), _ptr(out), n_requests, T, heads, dim, vdim, a2.shape[1], float(q_scale),
         1.0 / float(tau), float(eps), _stream()), "linear_recurrence_segments")
     return out
+
+
+SINK_DECODE_MAX_RUN = 128
+
+
+def sink_decode_supported(heads: int, kv_heads: int, dim: int, vdim: int) -> bool:
+    return bool(_load("sink_attention").cw_sink_decode_supported(heads, kv_heads, dim, vdim))
+
+
+def sink_attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, n_requests: int,
+                          run_keys: int, n_runs: int, r1, r2, sink, talk, heads: int, kv_heads: int, dim: int, vdim: int,
+                          block_size: int, window: int, scale: float) -> None:
+    """``sink_attention`` for the step's requests of one token each (others are left alone): the
+    keys a token sees are cut into ``n_runs`` runs of ``run_keys`` keys (the most any request of
+    the step has), a workgroup each; three kernels (scores and their sums, values, merge)."""
+    _gpu(q, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, r1, r2, sink, talk)
+    T = q.shape[0]
+    _need(q.dim() == 2 and q.shape[1] == q_stride and heads * dim <= q_stride, "q must be [T, q_stride] with the query heads first")
+    _need(tuple(out.shape) == (T, heads * vdim) and out.dtype == q.dtype, "out must be [T, heads * vdim]")
+    _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "cache and activations differ in type")
+    _need(tuple(k_cache.shape[-2:]) == (kv_heads, dim) and tuple(v_cache.shape[-2:]) == (kv_heads, vdim),
+          "the planes must be [..., kv_heads, dim] and [..., kv_heads, vdim]")
+    rows = k_cache.numel() // (kv_heads * dim)
+    _need(rows == v_cache.numel() // (kv_heads * vdim), "key and value planes must hold the same number of rows")
+    _i32(ctx_lens, n_requests, "ctx_lens")
+    _i32(cu_q, n_requests + 1, "cu_q")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= n_requests, "block tables must be int32 [R, width]")
+    for t, n, what in ((r1, heads, "r1"), (r2, heads, "r2"), (sink, heads, "sink"), (talk, heads * heads, "talk")):
+        _need(t is None or (t.dtype == torch.float32 and t.numel() == n), f"{what} must be float32 with {n} elements")
+    _need((r1 is None) == (r2 is None), "the distance bias takes r1 and r2 together")
+    _need(1 <= run_keys <= SINK_DECODE_MAX_RUN and n_runs >= 1, "runs of 1 to 128 keys, at least one")
+    lib = _load("sink_attention")
+    need = lib.cw_sink_decode_workspace_floats(n_requests, n_runs, run_keys, heads, vdim)
+    workspace = torch.empty(max(int(need), 1), dtype=torch.float32, device=q.device)
+    _check(lib.cw_sink_decode(
+        dtype_code(q.dtype), _ptr(q), q_stride, _ptr(out), _ptr(k_cache), _ptr(v_cache), rows, _ptr(block_tables),
+        block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), n_requests, run_keys, n_runs, _ptr(workspace), _ptr(r1), _ptr(r2),
+        _ptr(sink), _ptr(talk), heads, kv_heads, dim, vdim, block_size, int(window), float(scale), _stream()),
+        "sink_attention_decode")

@@ -3,8 +3,10 @@ sink in the softmax denominator and a mixing of the weights across heads (``Sink
 
 Steps: one fused q/k/v product; one kernel norms the query and key projections (float32
 statistics) and writes keys and values to their pages, so every token of the step is in the
-cache before any query reads it; the attention kernel reads the pages through the block table,
-prompt portions and single tokens in the same launch; output product. Keys and values have
+cache before any query reads it; the attention kernels read the pages through the block table:
+one launch for the step's prompt portions (a workgroup takes a run of a request's tokens with all
+heads), three small ones for its single tokens (a request's keys are shared among workgroups);
+output product. Keys and values have
 widths of their own, so the cache is two planes of a ``PagedRowsSpec``.
 """
 
@@ -19,15 +21,18 @@ from clockwork_amd.parts.base import EntryCache, Part
 from clockwork_amd.parts.specs import SinkAttentionSpec
 
 
-def query_runs(ctx, run: int):
+def query_runs(ctx, run: int, skip_single: bool = False):
     """The step's work items for a kernel whose workgroups take up to ``run`` consecutive tokens
     of one request with all heads: (request, first token, tokens, 0) each, uploaded once a step
-    and kept in ``ctx.plans``. Returns (device int32 array, number of items)."""
-    key = ("query runs", run)
+    and kept in ``ctx.plans``; ``skip_single``: requests of one token have a kernel of their own.
+    Returns (device int32 array, number of items)."""
+    key = ("query runs", run, skip_single)
     plan = ctx.plans.get(key)
     if plan is None:
         items = []
         for r, q_len in enumerate(ctx.h_q_lens):
+            if skip_single and q_len == 1:
+                continue
             tok0 = np.arange(0, q_len, run, dtype=np.int32)
             rows = np.zeros((tok0.size, 4), dtype=np.int32)
             rows[:, 0] = r
@@ -83,18 +88,37 @@ class SinkAttention(Part):
         self.sink, self.talk = params.get("sink"), params.get("talk")
         self.dtype = dtype
         self.run = ops.sink_attention_max_run(s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim)
+        self.decode_ok = ops.sink_decode_supported(s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim)
         if self.run < 1:
             raise ValueError(
                 f"attention with {s.num_heads} heads of {s.key_dim} / {s.value_dim} elements over {s.num_kv_heads} "
                 "key/value heads is beyond the sink-attention kernel (heads * value_dim up to 8192, 150 KB of LDS)")
 
-    def _runs(self, ctx):
-        # single tokens only: a run is one token; else the most the kernel takes
-        run = 1 if all(q == 1 for q in ctx.h_q_lens) else self.run
-        return run, query_runs(ctx, run)
+    def _plan(self, ctx):
+        """(items of the kernel for portions, their number, keys a run and runs of the kernels for
+        single tokens; 0 runs: the step has no single tokens, or they go with the portions)."""
+        key = ("sink attention", self.spec.window, self.decode_ok, self.run)
+        plan = ctx.plans.get(key)
+        if plan is None:
+            singles = [c for q, c in zip(ctx.h_q_lens, ctx.h_ctx_lens) if q == 1] if self.decode_ok else []
+            run_keys = n_runs = 0
+            if singles:
+                # the most keys a single token of this step sees, cut so that the workgroups about
+                # fill the card: runs of 32 to 128 keys
+                most = min(max(singles), self.spec.window or max(singles))
+                run_keys = 128
+                while run_keys > 32 and len(singles) * -(-most // run_keys) < ctx.num_compute_units:
+                    run_keys //= 2
+                n_runs = -(-most // run_keys)
+            items, n_items = query_runs(ctx, self.run, skip_single=bool(singles))
+            plan = ctx.plans[key] = (items, n_items, run_keys, n_runs)
+        return plan
 
     def prepare(self, ctx) -> None:
-        self._runs(ctx)
+        self._plan(ctx)
+
+    def shape_class(self, q_lens, ctx_lens):
+        return "single tokens" if all(q == 1 for q in q_lens) else "portions"
 
     def forward(self, x: torch.Tensor, ctx, cache: EntryCache) -> torch.Tensor:
         s = self.spec
@@ -106,8 +130,13 @@ class SinkAttention(Part):
         ops.qk_rownorm_store(qkv, 0, self.q_width, self.q_width + self.k_width, self.q_width, self.k_width, self.v_width,
                              self.q_norm, self.k_norm, s.qk_norm_eps, ctx.slots[cache.group], k_plane, v_plane)
         out = torch.empty((x.shape[0], s.num_heads * s.value_dim), dtype=x.dtype, device=x.device)
-        run, (items, n_items) = self._runs(ctx)
-        ops.sink_attention(qkv, qkv.shape[1], out, k_plane, v_plane, ctx.block_tables[cache.group], ctx.ctx_lens, ctx.cu_q,
-                           items, n_items, run, self.r1, self.r2, self.sink, self.talk, s.num_heads, s.num_kv_heads,
-                           s.key_dim, s.value_dim, cache.block_size, s.window or 0, s.scale)
+        items, n_items, run_keys, n_runs = self._plan(ctx)
+        options = (self.r1, self.r2, self.sink, self.talk, s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim,
+                   cache.block_size, s.window or 0, s.scale)
+        if n_items:
+            ops.sink_attention(qkv, qkv.shape[1], out, k_plane, v_plane, ctx.block_tables[cache.group], ctx.ctx_lens,
+                               ctx.cu_q, items, n_items, self.run, *options)
+        if n_runs:
+            ops.sink_attention_decode(qkv, qkv.shape[1], out, k_plane, v_plane, ctx.block_tables[cache.group], ctx.ctx_lens,
+                                      ctx.cu_q, ctx.num_requests, run_keys, n_runs, *options)
         return ops.linear(out, self.out_weight, policy=policy)
