@@ -566,3 +566,310 @@ CW_EXPORT int cw_sink_decode(int dtype, const void* q, int64_t q_stride, void* o
 #undef CW_LAUNCH
   return cw_launch_status();
 }
+
+// ======================================================================================
+// Portions in bfloat16 on the matrix cores. A workgroup owns 16 consecutive query tokens of one
+// request with ALL heads (the mixing across heads needs them together); its 4 waves share the
+// heads (wave w takes heads w, w + 4, ...). The keys are walked twice in chunks of 32, as in the
+// kernel above: first each row's maximum and denominator, then normalised weights, their mixing
+// across heads and the product with the values.
+//
+//   scores   S[16 q, 16 keys] = Q K^T     v_mfma_f32_16x16x32_bf16, Q fragments in registers for the
+//                                         whole kernel, K from an LDS tile shared by the waves;
+//   softmax  float32, on the lane's four rows of a tile; a row's statistics are finished across
+//            the 16 lanes that share it once, after the first walk, and stay in registers;
+//   mixing   the normalised weights of all heads meet in LDS as float32 [head][query][key]; a lane
+//            then makes, for each of its wave's heads, the 8 mixed weights that are its part of the
+//            next product's A operand;
+//   values   O[16 q, 16 dv] += P' V       P' is float32: it is fed as two bfloat16 operands, its
+//            leading 8 bits and the rounded rest, so the weights keep 16 bits of mantissa; V comes
+//            from an LDS tile that holds the chunk transposed, [dv][key].
+// ======================================================================================
+typedef __attribute__((ext_vector_type(8))) __bf16 sa_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float sa_f32x4_t;
+#define SM_KT 32
+#define SM_PROW 36   // floats a (head, query) row of weights takes in LDS: 32 and a pad against bank conflicts
+
+__device__ __forceinline__ sa_bf16x8_t sm_load8(const bf16_t* p) {
+  return *reinterpret_cast<const sa_bf16x8_t*>(p);
+}
+
+// HPW: heads a wave holds at most; D32: dim / 32; V16: vdim / 16
+template <int HPW, int D32, int V16>
+__global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  constexpr int D = D32 * 32, V = V16 * 16;
+  constexpr int KROW = D + 8;        // bf16 elements a key row takes in LDS
+  constexpr int VROW = SM_KT + 8;    // bf16 elements a value column takes in LDS
+  const int H = p.heads, G = p.kv_heads, Hg = H / G;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l16 = lane & 15, slot = lane >> 4;
+  const int r = p.items[4 * blockIdx.x], tok0 = p.items[4 * blockIdx.x + 1];
+  const int q_len = p.cu_q[r + 1] - p.cu_q[r];
+  if (tok0 >= q_len) return;
+  const int nq = min(min(p.items[4 * blockIdx.x + 2], 16), q_len - tok0);
+  const int pos0 = p.ctx_lens[r] - q_len + tok0;
+  const int last = pos0 + nq - 1;
+  const int lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
+  const int64_t row0 = p.cu_q[r] + tok0;
+  const int* table = p.block_tables + (int64_t)r * p.table_width;
+
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(smem_raw);              // [G][KT][KROW]
+  bf16_t* Vt = Ks + G * SM_KT * KROW;                            // [G][V][VROW]
+  float* Pn = reinterpret_cast<float*>(Vt + G * V * VROW);       // [H][16][SM_PROW]
+  float* Tk = Pn + H * 16 * SM_PROW;                             // [H][H]
+
+  const bf16_t* q = (const bf16_t*)p.q;
+  const bf16_t* kc = (const bf16_t*)p.k_cache;
+  const bf16_t* vc = (const bf16_t*)p.v_cache;
+  if (p.talk)
+    for (int i = tid; i < H * H; i += 256) Tk[i] = p.talk[i];
+
+  // this wave's heads and their query fragments: lane = query l16, 8 elements at slot
+  sa_bf16x8_t qf[HPW][D32];
+  const int qi = min(l16, nq - 1);
+#pragma unroll
+  for (int a = 0; a < HPW; ++a) {
+    const int g = min(wave + 4 * a, H - 1);
+#pragma unroll
+    for (int ks = 0; ks < D32; ++ks) qf[a][ks] = sm_load8(q + (row0 + qi) * p.q_stride + g * D + ks * 32 + slot * 8);
+  }
+
+  // the chunk's keys of every key/value head into LDS; keys past ``last`` or without a page: zeros
+  auto load_keys = [&](int k0) {
+    constexpr int PER_ROW = D / 8;
+    for (int idx = tid; idx < G * SM_KT * PER_ROW; idx += 256) {
+      const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
+      const int j = k0 + jj;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (j <= last) {
+        const int page = table[j / p.block_size];
+        const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
+        if (page >= 0 && row < p.cache_rows) v = *reinterpret_cast<const uint4*>(kc + (row * G + c) * D + e * 8);
+      }
+      *reinterpret_cast<uint4*>(Ks + (c * SM_KT + jj) * KROW + e * 8) = v;
+    }
+  };
+  auto load_values = [&](int k0) {
+    constexpr int PER_ROW = V / 8;
+    for (int idx = tid; idx < G * SM_KT * PER_ROW; idx += 256) {
+      const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
+      const int j = k0 + jj;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (j <= last) {
+        const int page = table[j / p.block_size];
+        const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
+        if (page >= 0 && row < p.cache_rows) v = *reinterpret_cast<const uint4*>(vc + (row * G + c) * V + e * 8);
+      }
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      uint16_t* dst = reinterpret_cast<uint16_t*>(Vt) + (c * V + e * 8) * VROW + jj;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        dst[(2 * u) * VROW] = (uint16_t)(w[u] & 0xffffu);
+        dst[(2 * u + 1) * VROW] = (uint16_t)(w[u] >> 16);
+      }
+    }
+  };
+  // the scores of head g's tile kt of the chunk: rows slot * 4 + e, key 16 kt + l16; -inf where not seen
+  auto scores = [&](int a, int g, int kt, int k0, float* s) {
+    const int c = g / Hg;
+    sa_f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bf16_t* kb = Ks + (c * SM_KT + kt * 16 + l16) * KROW + slot * 8;
+#pragma unroll
+    for (int ks = 0; ks < D32; ++ks)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[a][ks], sm_load8(kb + ks * 32), acc, 0, 0, 0);
+    const int j = k0 + kt * 16 + l16;
+    const float r1 = p.r1 ? p.r1[g] : 0.0f, r2 = p.r1 ? p.r2[g] : 0.0f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int i = slot * 4 + e;
+      const int dist = pos0 + i - j;
+      float v = acc[e] * p.scale;
+      if (p.r1) v -= r1 * __logf(1.0f + r2 * (float)max(dist, 0));
+      const bool seen = i < nq && dist >= 0 && (p.window <= 0 || dist < p.window);
+      s[e] = seen ? v : -INFINITY;
+    }
+  };
+
+  // ---- first walk: maxima and denominators, per lane, then across the 16 lanes of a row
+  float m[HPW][4], l[HPW][4];
+#pragma unroll
+  for (int a = 0; a < HPW; ++a) {
+    const int g = min(wave + 4 * a, H - 1);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      m[a][e] = p.sink ? p.sink[g] : -3.0e38f;
+      l[a][e] = (p.sink && l16 == 0) ? 1.0f : 0.0f;
+    }
+  }
+  for (int k0 = lo; k0 <= last; k0 += SM_KT) {
+    __syncthreads();
+    load_keys(k0);
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < HPW; ++a) {
+      const int g = wave + 4 * a;
+      if (g < H) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+          float s[4];
+          scores(a, g, kt, k0, s);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float mn = fmaxf(m[a][e], s[e]);
+            l[a][e] = l[a][e] * __expf(m[a][e] - mn) + __expf(s[e] - mn);
+            m[a][e] = mn;
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < HPW; ++a)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) {
+        const float mo = __shfl_xor(m[a][e], off, 16), lo_ = __shfl_xor(l[a][e], off, 16);
+        const float mn = fmaxf(m[a][e], mo);
+        l[a][e] = l[a][e] * __expf(m[a][e] - mn) + lo_ * __expf(mo - mn);
+        m[a][e] = mn;
+      }
+      l[a][e] = l[a][e] > 0.0f ? 1.0f / l[a][e] : 0.0f;  // from here on: 1 / denominator
+    }
+
+  // ---- second walk
+  sa_f32x4_t out[HPW][V16];
+#pragma unroll
+  for (int a = 0; a < HPW; ++a)
+#pragma unroll
+    for (int nt = 0; nt < V16; ++nt) out[a][nt] = sa_f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int k0 = lo; k0 <= last; k0 += SM_KT) {
+    __syncthreads();
+    load_keys(k0);
+    load_values(k0);
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < HPW; ++a) {
+      const int g = wave + 4 * a;
+      if (g < H) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+          float s[4];
+          scores(a, g, kt, k0, s);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            Pn[(g * 16 + slot * 4 + e) * SM_PROW + kt * 16 + l16] = __expf(s[e] - m[a][e]) * l[a][e];
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < HPW; ++a) {
+      const int h = wave + 4 * a;
+      if (h < H) {
+        // this lane's part of the A operand: query l16, keys slot * 8 .. + 8 of the chunk
+        float w[8];
+        if (p.talk) {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) w[u] = 0.0f;
+          for (int g = 0; g < H; ++g) {
+            const float t = Tk[h * H + g];
+            const float4 x = *reinterpret_cast<const float4*>(Pn + (g * 16 + l16) * SM_PROW + slot * 8);
+            const float4 y = *reinterpret_cast<const float4*>(Pn + (g * 16 + l16) * SM_PROW + slot * 8 + 4);
+            w[0] += t * x.x; w[1] += t * x.y; w[2] += t * x.z; w[3] += t * x.w;
+            w[4] += t * y.x; w[5] += t * y.y; w[6] += t * y.z; w[7] += t * y.w;
+          }
+        } else {
+          const float4 x = *reinterpret_cast<const float4*>(Pn + (h * 16 + l16) * SM_PROW + slot * 8);
+          const float4 y = *reinterpret_cast<const float4*>(Pn + (h * 16 + l16) * SM_PROW + slot * 8 + 4);
+          w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w; w[4] = y.x; w[5] = y.y; w[6] = y.z; w[7] = y.w;
+        }
+        sa_bf16x8_t hi, lo8;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const __bf16 top = (__bf16)w[u];
+          hi[u] = top;
+          lo8[u] = (__bf16)(w[u] - (float)top);
+        }
+        const int c = h / Hg;
+        const bf16_t* vb = Vt + (c * V + l16) * VROW + slot * 8;
+#pragma unroll
+        for (int nt = 0; nt < V16; ++nt) {
+          const sa_bf16x8_t vf = sm_load8(vb + nt * 16 * VROW);
+          out[a][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, vf, out[a][nt], 0, 0, 0);
+          out[a][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lo8, vf, out[a][nt], 0, 0, 0);
+        }
+      }
+    }
+  }
+  bf16_t* o = (bf16_t*)p.out;
+#pragma unroll
+  for (int a = 0; a < HPW; ++a) {
+    const int h = wave + 4 * a;
+    if (h < H) {
+#pragma unroll
+      for (int nt = 0; nt < V16; ++nt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = slot * 4 + e;
+          if (i < nq) o[(row0 + i) * (int64_t)(H * V) + h * V + nt * 16 + l16] = __float2bfloat16(out[a][nt][e]);
+        }
+    }
+  }
+}
+
+static int64_t sink_prefill_mfma_lds_bytes(int H, int G, int D, int V) {
+  return (int64_t)G * SM_KT * (D + 8) * 2 + (int64_t)G * V * (SM_KT + 8) * 2 + (int64_t)H * 16 * SM_PROW * 4 + (int64_t)H * H * 4;
+}
+
+// The geometries this kernel is built for: dim 64 or 128, vdim 64 or 128, up to 16 heads
+// (4 a wave), and what of LDS they need.
+CW_EXPORT int cw_sink_prefill_mfma_supported(int heads, int kv_heads, int dim, int vdim) {
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || heads > 16) return 0;
+  if ((dim != 64 && dim != 128) || (vdim != 64 && vdim != 128)) return 0;
+  return sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim) <= 150 * 1024 ? 1 : 0;
+}
+
+// items: runs of up to 16 tokens. bfloat16 only.
+CW_EXPORT int cw_sink_prefill_mfma(const void* q, int64_t q_stride, void* out, const void* k_cache, const void* v_cache,
+                                   int64_t cache_rows, const int* block_tables, int table_width, const int* ctx_lens,
+                                   const int* cu_q, const int* items, int n_items, const float* r1, const float* r2,
+                                   const float* sink, const float* talk, int heads, int kv_heads, int dim, int vdim,
+                                   int block_size, int window, float scale, hipStream_t stream) {
+  if (n_items < 0 || !q || !out || !k_cache || !v_cache || !block_tables || !ctx_lens || !cu_q || !items) return CW_ERR_ARG;
+  if (block_size <= 0 || table_width <= 0 || window < 0 || (r1 && !r2)) return CW_ERR_ARG;
+  if (!cw_sink_prefill_mfma_supported(heads, kv_heads, dim, vdim)) return CW_ERR_SIZE;
+  if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || (q_stride % 8)) return CW_ERR_ARG;
+  if (n_items == 0) return CW_OK;
+  SinkAttnParams p;
+  p.q = q; p.q_stride = q_stride; p.out = out; p.k_cache = k_cache; p.v_cache = v_cache;
+  p.block_tables = block_tables; p.table_width = table_width; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
+  p.r1 = r1; p.r2 = r2; p.sink = sink; p.talk = talk;
+  p.heads = heads; p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.block_size = block_size; p.window = window;
+  p.scale = scale; p.bq = 16; p.cache_rows = cache_rows;
+  const size_t smem = (size_t)sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim);
+  const dim3 grid(n_items), block(256);
+  const int hpw = (heads + 3) / 4;
+#define CW_LAUNCH(HPW_, D32_, V16_)                                                                                   \
+  do {                                                                                                                \
+    if (smem > 48 * 1024 && hipFuncSetAttribute((const void*)sink_prefill_mfma_kernel<HPW_, D32_, V16_>,              \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) \
+      return CW_ERR_LAUNCH;                                                                                           \
+    hipLaunchKernelGGL((sink_prefill_mfma_kernel<HPW_, D32_, V16_>), grid, block, smem, stream, p);                   \
+  } while (0)
+#define CW_BY_HEADS(D32_, V16_)                \
+  do {                                         \
+    if (hpw <= 1) CW_LAUNCH(1, D32_, V16_);    \
+    else if (hpw == 2) CW_LAUNCH(2, D32_, V16_); \
+    else if (hpw == 3) CW_LAUNCH(3, D32_, V16_); \
+    else CW_LAUNCH(4, D32_, V16_);             \
+  } while (0)
+  if (dim == 64 && vdim == 64) CW_BY_HEADS(2, 4);
+  else if (dim == 64 && vdim == 128) CW_BY_HEADS(2, 8);
+  else if (dim == 128 && vdim == 64) CW_BY_HEADS(4, 4);
+  else CW_BY_HEADS(4, 8);
+#undef CW_BY_HEADS
+#undef CW_LAUNCH
+  return cw_launch_status();
+}

@@ -131,6 +131,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_sink_attention_max_bq": [I, I, I, I],
             "cw_sink_attention": [I, P, L, P, P, P, L, P, I, P, P, P, I, I, P, P, P, P, I, I, I, I, I, I, F, P],
             "cw_sink_decode_workspace_floats": [I, I, I, I, I],
+            "cw_sink_prefill_mfma_supported": [I, I, I, I],
+            "cw_sink_prefill_mfma": [P, L, P, P, P, L, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, P],
             "cw_sink_decode_supported": [I, I, I, I],
             "cw_sink_decode": [I, P, L, P, P, P, L, P, I, P, P, I, I, I, P, P, P, P, P, I, I, I, I, I, I, F, P],
         },
@@ -1503,3 +1505,39 @@ def sink_attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables,
         block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), n_requests, run_keys, n_runs, _ptr(workspace), _ptr(r1), _ptr(r2),
         _ptr(sink), _ptr(talk), heads, kv_heads, dim, vdim, block_size, int(window), float(scale), _stream()),
         "sink_attention_decode")
+
+
+def sink_prefill_mfma_supported(heads: int, kv_heads: int, dim: int, vdim: int, dtype) -> bool:
+    """Is there a matrix-core build of the sink-attention kernel for portions of this geometry?
+    (bfloat16; key and value sizes of 64 or 128; up to 16 heads.)"""
+    return dtype == torch.bfloat16 and bool(_load("sink_attention").cw_sink_prefill_mfma_supported(heads, kv_heads, dim, vdim))
+
+
+def sink_attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
+                           r1, r2, sink, talk, heads: int, kv_heads: int, dim: int, vdim: int, block_size: int, window: int,
+                           scale: float) -> None:
+    """``sink_attention`` on the matrix cores for bfloat16 portions: ``items`` are runs of up to
+    16 tokens. Scores, softmax and the mixing across heads are float32; the mixed weights meet
+    the values as two bfloat16 operands (leading bits and rest)."""
+    _gpu(q, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, r1, r2, sink, talk)
+    T = q.shape[0]
+    _need(q.dtype == torch.bfloat16 and q.dim() == 2 and q.shape[1] == q_stride and heads * dim <= q_stride and q_stride % 8 == 0,
+          "q must be bfloat16 [T, q_stride], q_stride a multiple of 8, with the query heads first")
+    _need(tuple(out.shape) == (T, heads * vdim) and out.dtype == q.dtype, "out must be [T, heads * vdim]")
+    _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "cache and activations differ in type")
+    _need(tuple(k_cache.shape[-2:]) == (kv_heads, dim) and tuple(v_cache.shape[-2:]) == (kv_heads, vdim),
+          "the planes must be [..., kv_heads, dim] and [..., kv_heads, vdim]")
+    rows = k_cache.numel() // (kv_heads * dim)
+    _need(rows == v_cache.numel() // (kv_heads * vdim), "key and value planes must hold the same number of rows")
+    R = ctx_lens.numel()
+    _i32(ctx_lens, R, "ctx_lens")
+    _i32(cu_q, R + 1, "cu_q")
+    _i32(items, 4 * n_items, "items")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= R, "block tables must be int32 [R, width]")
+    for t, n, what in ((r1, heads, "r1"), (r2, heads, "r2"), (sink, heads, "sink"), (talk, heads * heads, "talk")):
+        _need(t is None or (t.dtype == torch.float32 and t.numel() == n), f"{what} must be float32 with {n} elements")
+    _need((r1 is None) == (r2 is None), "the distance bias takes r1 and r2 together")
+    _check(_load("sink_attention").cw_sink_prefill_mfma(
+        _ptr(q), q_stride, _ptr(out), _ptr(k_cache), _ptr(v_cache), rows, _ptr(block_tables), block_tables.shape[1],
+        _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(r1), _ptr(r2), _ptr(sink), _ptr(talk), heads, kv_heads, dim,
+        vdim, block_size, int(window), float(scale), _stream()), "sink_attention_prefill")

@@ -88,6 +88,9 @@ class SinkAttention(Part):
         self.sink, self.talk = params.get("sink"), params.get("talk")
         self.dtype = dtype
         self.run = ops.sink_attention_max_run(s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim)
+        # bfloat16 portions of the common head sizes run on the matrix cores; the kernel reads 16 bytes at a time
+        self.mfma_ok = (ops.sink_prefill_mfma_supported(s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim, dtype)
+                        and (self.q_width + self.k_width + self.v_width) % 8 == 0)
         self.decode_ok = ops.sink_decode_supported(s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim)
         if self.run < 1:
             raise ValueError(
@@ -97,7 +100,7 @@ class SinkAttention(Part):
     def _plan(self, ctx):
         """(items of the kernel for portions, their number, keys a run and runs of the kernels for
         single tokens; 0 runs: the step has no single tokens, or they go with the portions)."""
-        key = ("sink attention", self.spec.window, self.decode_ok, self.run)
+        key = ("sink attention", self.spec.window, self.decode_ok, self.run, self.mfma_ok)
         plan = ctx.plans.get(key)
         if plan is None:
             singles = [c for q, c in zip(ctx.h_q_lens, ctx.h_ctx_lens) if q == 1] if self.decode_ok else []
@@ -110,7 +113,7 @@ class SinkAttention(Part):
                 while run_keys > 32 and len(singles) * -(-most // run_keys) < ctx.num_compute_units:
                     run_keys //= 2
                 n_runs = -(-most // run_keys)
-            items, n_items = query_runs(ctx, self.run, skip_single=bool(singles))
+            items, n_items = query_runs(ctx, 16 if self.mfma_ok else self.run, skip_single=bool(singles))
             plan = ctx.plans[key] = (items, n_items, run_keys, n_runs)
         return plan
 
@@ -133,7 +136,10 @@ class SinkAttention(Part):
         items, n_items, run_keys, n_runs = self._plan(ctx)
         options = (self.r1, self.r2, self.sink, self.talk, s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim,
                    cache.block_size, s.window or 0, s.scale)
-        if n_items:
+        if n_items and self.mfma_ok:
+            ops.sink_attention_prefill(qkv, qkv.shape[1], out, k_plane, v_plane, ctx.block_tables[cache.group], ctx.ctx_lens,
+                                       ctx.cu_q, items, n_items, *options)
+        elif n_items:
             ops.sink_attention(qkv, qkv.shape[1], out, k_plane, v_plane, ctx.block_tables[cache.group], ctx.ctx_lens,
                                ctx.cu_q, items, n_items, self.run, *options)
         if n_runs:

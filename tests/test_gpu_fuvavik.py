@@ -197,6 +197,11 @@ LEFT_SHAPES = [
     (3, 1, 40, 24, 300, 50),
     (1, 1, 8, 72, 1, 40),
     (16, 4, 64, 32, 20, 96),
+    # the sizes that the matrix-core kernel for bfloat16 portions takes
+    (12, 2, 128, 128, 40, 64),
+    (6, 3, 64, 128, 23, 48),
+    (16, 16, 128, 64, 300, 32),
+    (1, 1, 64, 64, 7, 40),
 ]
 
 
@@ -214,6 +219,27 @@ def test_sink_attention_whole_in_portions_and_token_by_token(dtype, shape):
     for cuts in ([T], [5, 1, 1, 17, 2, 1, 2, 32], [1] * T):
         got = _step_through(part, part.cache_need(), x, cuts, dtype)
         close(got, want, dtype)
+    if part.mfma_ok:
+        # the matrix-core kernel against the plain-arithmetic one on the very same bfloat16 queries,
+        # keys and values: they differ by the order of their sums and the rounding of the output
+        # alone, a tenth of what separates either from the float64 result
+        assert dtype == torch.bfloat16
+        fast = _step_through(part, part.cache_need(), x, [T], dtype)
+        part.mfma_ok = False
+        slow = _step_through(part, part.cache_need(), x, [T], dtype)
+        scale = float(want.square().mean().sqrt())
+        assert float((fast - slow).abs().max()) < 1.5e-2 * scale and float((fast - slow).square().mean().sqrt()) < 3e-3 * scale
+
+
+def test_the_matrix_core_kernel_is_the_one_that_runs_for_bfloat16_portions():
+    spec = SinkAttentionSpec(hidden_size=64, num_heads=12, num_kv_heads=2, key_dim=128, value_dim=128, scale=0.1, window=40)
+    for dtype, expected in ((torch.bfloat16, True), (torch.float32, False)):
+        part = build_part(spec)
+        bind(part, dtype)
+        assert part.mfma_ok is expected and part.decode_ok
+    odd = build_part(SinkAttentionSpec(hidden_size=64, num_heads=4, num_kv_heads=2, key_dim=24, value_dim=16, scale=0.1, window=9))
+    bind(odd, torch.bfloat16)
+    assert not odd.mfma_ok and odd.run >= 1
 
 
 def test_sink_attention_options_each_matter():
