@@ -548,7 +548,9 @@ __global__ void fresh_state_rows_kernel(uint32_t* __restrict__ pool, int64_t ent
   if (starts[r] != 0 || slot < 0 || slot >= num_slots) return;
   uint32_t* row = pool + entry * entry_words + (int64_t)slot * row_words;
   const uint32_t* fresh = pool + entry * entry_words + (int64_t)fresh_slot * row_words;
-  for (int64_t i = threadIdx.x; i < row_words; i += blockDim.x) row[i] = fresh[i];
+  // a large state (a matrix per head) is shared among the workgroups of gridDim.z
+  for (int64_t i = (int64_t)blockIdx.z * blockDim.x + threadIdx.x; i < row_words; i += (int64_t)gridDim.z * blockDim.x)
+    row[i] = fresh[i];
 }
 
 // pool [entries, pool_slots, row_bytes]: slots [0, num_slots) may be set, slot ``fresh_slot`` (one of
@@ -560,7 +562,9 @@ CW_EXPORT int cw_fresh_state_rows(void* pool, int entries, int pool_slots, int n
   if (num_slots > pool_slots || fresh_slot < num_slots || fresh_slot >= pool_slots) return CW_ERR_ARG;
   if (n == 0) return CW_OK;
   if (entries > 65535) return CW_ERR_SIZE;
-  hipLaunchKernelGGL(fresh_state_rows_kernel, dim3(n, entries), dim3(256), 0, stream, (uint32_t*)pool,
+  int64_t parts = (row_bytes / 4 + 4095) / 4096;  // about sixteen words a thread
+  if (parts > 64) parts = 64;
+  hipLaunchKernelGGL(fresh_state_rows_kernel, dim3(n, entries, (unsigned)parts), dim3(256), 0, stream, (uint32_t*)pool,
                      (int64_t)pool_slots * (row_bytes / 4), row_bytes / 4, num_slots, fresh_slot, slots, starts);
   return cw_launch_status();
 }

@@ -226,19 +226,50 @@ struct SegParams {
   float q_scale, inv_tau, eps;
 };
 
+template <typename T> struct LrVec;
+template <> struct LrVec<float> {
+  static constexpr int N = 4;
+  __device__ static void load(const float* p, float* o) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+  }
+};
+template <> struct LrVec<bf16_t> {
+  static constexpr int N = 8;
+  __device__ static void load(const bf16_t* p, float* o) {
+    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(w[i] << 16); o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+  }
+};
+
 template <typename T>
 __global__ __launch_bounds__(256) void lrs_prepare_kernel(SegParams p) {
   const int HD = p.heads * p.dim;
   const int64_t n = (int64_t)p.n_tokens * HD;
   const T* proj = (const T*)p.proj;
   const T* a2 = (const T*)p.a2;
+  constexpr int N = LrVec<T>::N;
+  const bool vec = p.rank % N == 0 && p.u_off % N == 0 && p.stride % N == 0 && !((uintptr_t)proj & 15) && !((uintptr_t)a2 & 15);
   for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * 256) {
     const int64_t t = idx / HD;
     const int c = (int)(idx - t * HD);
     const T* row = proj + t * p.stride;
     float z = p.a2b ? p.a2b[c] : 0.0f;
     const T* w = a2 + (int64_t)c * p.rank;
-    for (int e = 0; e < p.rank; ++e) z += cw_to_float(w[e]) * cw_to_float(row[p.u_off + e]);
+    const T* u = row + p.u_off;
+    if (vec) {  // 16 bytes of the decay matrix's row and of the token's decay input at a time
+      for (int e = 0; e < p.rank; e += N) {
+        float wv[N], uv[N];
+        LrVec<T>::load(w + e, wv);
+        LrVec<T>::load(u + e, uv);
+#pragma unroll
+        for (int i = 0; i < N; ++i) z += wv[i] * uv[i];
+      }
+    } else {
+      for (int e = 0; e < p.rank; ++e) z += cw_to_float(w[e]) * cw_to_float(u[e]);
+    }
     const float ls = z < 0.0f ? z - log1pf(expf(z)) : -log1pf(expf(-z));
     p.dec[idx] = expf(ls * p.inv_tau);
     p.qf[idx] = cw_to_float(row[p.q_off + c]) * p.q_scale;

@@ -428,14 +428,21 @@ __global__ __launch_bounds__(256) void sink_decode_values_kernel(SinkDecodeParam
   float* mg = Pm + H * SK;       // [H] maxima
   float* il = mg + H;            // [H] 1 / denominators
   int* rows = (int*)(il + H);    // [SK] cache rows of the run's keys (-1: none)
-  for (int g = tid; g < H; g += 256) {
-    float m = p.sink ? p.sink[g] : -INFINITY;
+  // every head's final maximum and denominator from the runs' own: a wave per head, a lane per run
+  for (int g = tid >> 6; g < H; g += 4) {
+    const int ln = tid & 63;
     const float* st = p.stats + ((int64_t)r * p.n_runs * H + g) * 2;
-    for (int s = 0; s < runs; ++s) m = fmaxf(m, st[(int64_t)s * H * 2]);
-    float l = p.sink ? expf(p.sink[g] - m) : 0.0f;
-    for (int s = 0; s < runs; ++s) l += st[(int64_t)s * H * 2 + 1] * expf(st[(int64_t)s * H * 2] - m);
-    mg[g] = m;
-    il[g] = l > 0.0f ? 1.0f / l : 0.0f;
+    float m = p.sink ? p.sink[g] : -INFINITY;
+    for (int s = ln; s < runs; s += 64) m = fmaxf(m, st[(int64_t)s * H * 2]);
+    m = cw_wave_max(m);
+    float l = 0.0f;
+    for (int s = ln; s < runs; s += 64) l += st[(int64_t)s * H * 2 + 1] * expf(st[(int64_t)s * H * 2] - m);
+    l = cw_wave_sum(l);
+    if (p.sink) l += expf(p.sink[g] - m);
+    if (ln == 0) {
+      mg[g] = m;
+      il[g] = l > 0.0f ? 1.0f / l : 0.0f;
+    }
   }
   const int* table = p.block_tables + (int64_t)r * p.table_width;
   for (int jj = tid; jj < SK; jj += 256) {
@@ -594,11 +601,14 @@ __device__ __forceinline__ sa_bf16x8_t sm_load8(const bf16_t* p) {
   return *reinterpret_cast<const sa_bf16x8_t*>(p);
 }
 
-// HPW: heads a wave holds at most; D32: dim / 32; V16: vdim / 16
-template <int HPW, int D32, int V16>
+// HPW: heads a wave holds at most; D32: dim / 32; V16: vdim / 16; VS: workgroups that share a run's
+// value columns (blockIdx.y: each makes all the weights and its own V16 / VS column tiles of the
+// output; a launch of few runs fills the card that way)
+template <int HPW, int D32, int V16, int VS>
 __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  constexpr int D = D32 * 32, V = V16 * 16;
+  constexpr int D = D32 * 32, V = V16 * 16, NT = V16 / VS, VW = NT * 16;
+  const int v0 = blockIdx.y * VW;   // this workgroup's first value column
   constexpr int KROW = D + 8;        // bf16 elements a key row takes in LDS
   constexpr int VROW = SM_KT + 8;    // bf16 elements a value column takes in LDS
   const int H = p.heads, G = p.kv_heads, Hg = H / G;
@@ -615,8 +625,8 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
   const int* table = p.block_tables + (int64_t)r * p.table_width;
 
   bf16_t* Ks = reinterpret_cast<bf16_t*>(smem_raw);              // [G][KT][KROW]
-  bf16_t* Vt = Ks + G * SM_KT * KROW;                            // [G][V][VROW]
-  float* Pn = reinterpret_cast<float*>(Vt + G * V * VROW);       // [H][16][SM_PROW]
+  bf16_t* Vt = Ks + G * SM_KT * KROW;                            // [G][VW][VROW]
+  float* Pn = reinterpret_cast<float*>(Vt + G * VW * VROW);      // [H][16][SM_PROW]
   float* Tk = Pn + H * 16 * SM_PROW;                             // [H][H]
 
   const bf16_t* q = (const bf16_t*)p.q;
@@ -651,7 +661,7 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
     }
   };
   auto load_values = [&](int k0) {
-    constexpr int PER_ROW = V / 8;
+    constexpr int PER_ROW = VW / 8;
     for (int idx = tid; idx < G * SM_KT * PER_ROW; idx += 256) {
       const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
       const int j = k0 + jj;
@@ -659,10 +669,10 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
       if (j <= last) {
         const int page = table[j / p.block_size];
         const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
-        if (page >= 0 && row < p.cache_rows) v = *reinterpret_cast<const uint4*>(vc + (row * G + c) * V + e * 8);
+        if (page >= 0 && row < p.cache_rows) v = *reinterpret_cast<const uint4*>(vc + (row * G + c) * V + v0 + e * 8);
       }
       const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-      uint16_t* dst = reinterpret_cast<uint16_t*>(Vt) + (c * V + e * 8) * VROW + jj;
+      uint16_t* dst = reinterpret_cast<uint16_t*>(Vt) + (c * VW + e * 8) * VROW + jj;
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         dst[(2 * u) * VROW] = (uint16_t)(w[u] & 0xffffu);
@@ -739,11 +749,11 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
     }
 
   // ---- second walk
-  sa_f32x4_t out[HPW][V16];
+  sa_f32x4_t out[HPW][NT];
 #pragma unroll
   for (int a = 0; a < HPW; ++a)
 #pragma unroll
-    for (int nt = 0; nt < V16; ++nt) out[a][nt] = sa_f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int nt = 0; nt < NT; ++nt) out[a][nt] = sa_f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
   for (int k0 = lo; k0 <= last; k0 += SM_KT) {
     __syncthreads();
     load_keys(k0);
@@ -793,9 +803,9 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
           lo8[u] = (__bf16)(w[u] - (float)top);
         }
         const int c = h / Hg;
-        const bf16_t* vb = Vt + (c * V + l16) * VROW + slot * 8;
+        const bf16_t* vb = Vt + (c * VW + l16) * VROW + slot * 8;
 #pragma unroll
-        for (int nt = 0; nt < V16; ++nt) {
+        for (int nt = 0; nt < NT; ++nt) {
           const sa_bf16x8_t vf = sm_load8(vb + nt * 16 * VROW);
           out[a][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, vf, out[a][nt], 0, 0, 0);
           out[a][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lo8, vf, out[a][nt], 0, 0, 0);
@@ -809,17 +819,17 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
     const int h = wave + 4 * a;
     if (h < H) {
 #pragma unroll
-      for (int nt = 0; nt < V16; ++nt)
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int i = slot * 4 + e;
-          if (i < nq) o[(row0 + i) * (int64_t)(H * V) + h * V + nt * 16 + l16] = __float2bfloat16(out[a][nt][e]);
+          if (i < nq) o[(row0 + i) * (int64_t)(H * V) + h * V + v0 + nt * 16 + l16] = __float2bfloat16(out[a][nt][e]);
         }
     }
   }
 }
 
-static int64_t sink_prefill_mfma_lds_bytes(int H, int G, int D, int V) {
+static int64_t sink_prefill_mfma_lds_bytes(int H, int G, int D, int V) {  // V: the value columns of one workgroup
   return (int64_t)G * SM_KT * (D + 8) * 2 + (int64_t)G * V * (SM_KT + 8) * 2 + (int64_t)H * 16 * SM_PROW * 4 + (int64_t)H * H * 4;
 }
 
@@ -831,12 +841,13 @@ CW_EXPORT int cw_sink_prefill_mfma_supported(int heads, int kv_heads, int dim, i
   return sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim) <= 150 * 1024 ? 1 : 0;
 }
 
-// items: runs of up to 16 tokens. bfloat16 only.
+// items: runs of up to 16 tokens. bfloat16 only. A launch of fewer than v_split_below runs gives
+// every run two workgroups (the caller passes the number of compute units).
 CW_EXPORT int cw_sink_prefill_mfma(const void* q, int64_t q_stride, void* out, const void* k_cache, const void* v_cache,
                                    int64_t cache_rows, const int* block_tables, int table_width, const int* ctx_lens,
                                    const int* cu_q, const int* items, int n_items, const float* r1, const float* r2,
                                    const float* sink, const float* talk, int heads, int kv_heads, int dim, int vdim,
-                                   int block_size, int window, float scale, hipStream_t stream) {
+                                   int block_size, int window, float scale, int v_split_below, hipStream_t stream) {
   if (n_items < 0 || !q || !out || !k_cache || !v_cache || !block_tables || !ctx_lens || !cu_q || !items) return CW_ERR_ARG;
   if (block_size <= 0 || table_width <= 0 || window < 0 || (r1 && !r2)) return CW_ERR_ARG;
   if (!cw_sink_prefill_mfma_supported(heads, kv_heads, dim, vdim)) return CW_ERR_SIZE;
@@ -848,15 +859,22 @@ CW_EXPORT int cw_sink_prefill_mfma(const void* q, int64_t q_stride, void* out, c
   p.r1 = r1; p.r2 = r2; p.sink = sink; p.talk = talk;
   p.heads = heads; p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.block_size = block_size; p.window = window;
   p.scale = scale; p.bq = 16; p.cache_rows = cache_rows;
-  const size_t smem = (size_t)sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim);
-  const dim3 grid(n_items), block(256);
+  // few runs: two workgroups a run, each with half of the value columns
+  const int vs = n_items < v_split_below ? 2 : 1;
+  const size_t smem = (size_t)sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim / vs);
+  const dim3 grid(n_items, vs), block(256);
   const int hpw = (heads + 3) / 4;
-#define CW_LAUNCH(HPW_, D32_, V16_)                                                                                   \
+#define CW_LAUNCH_VS(HPW_, D32_, V16_, VS_)                                                                           \
   do {                                                                                                                \
-    if (smem > 48 * 1024 && hipFuncSetAttribute((const void*)sink_prefill_mfma_kernel<HPW_, D32_, V16_>,              \
+    if (smem > 48 * 1024 && hipFuncSetAttribute((const void*)sink_prefill_mfma_kernel<HPW_, D32_, V16_, VS_>,         \
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) \
       return CW_ERR_LAUNCH;                                                                                           \
-    hipLaunchKernelGGL((sink_prefill_mfma_kernel<HPW_, D32_, V16_>), grid, block, smem, stream, p);                   \
+    hipLaunchKernelGGL((sink_prefill_mfma_kernel<HPW_, D32_, V16_, VS_>), grid, block, smem, stream, p);              \
+  } while (0)
+#define CW_LAUNCH(HPW_, D32_, V16_)                 \
+  do {                                              \
+    if (vs == 2) CW_LAUNCH_VS(HPW_, D32_, V16_, 2); \
+    else CW_LAUNCH_VS(HPW_, D32_, V16_, 1);         \
   } while (0)
 #define CW_BY_HEADS(D32_, V16_)                \
   do {                                         \
@@ -871,5 +889,6 @@ CW_EXPORT int cw_sink_prefill_mfma(const void* q, int64_t q_stride, void* out, c
   else CW_BY_HEADS(4, 8);
 #undef CW_BY_HEADS
 #undef CW_LAUNCH
+#undef CW_LAUNCH_VS
   return cw_launch_status();
 }

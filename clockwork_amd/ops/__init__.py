@@ -132,7 +132,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_sink_attention": [I, P, L, P, P, P, L, P, I, P, P, P, I, I, P, P, P, P, I, I, I, I, I, I, F, P],
             "cw_sink_decode_workspace_floats": [I, I, I, I, I],
             "cw_sink_prefill_mfma_supported": [I, I, I, I],
-            "cw_sink_prefill_mfma": [P, L, P, P, P, L, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, P],
+            "cw_sink_prefill_mfma": [P, L, P, P, P, L, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, P],
             "cw_sink_decode_supported": [I, I, I, I],
             "cw_sink_decode": [I, P, L, P, P, P, L, P, I, P, P, I, I, I, P, P, P, P, P, I, I, I, I, I, I, F, P],
         },
@@ -1515,9 +1515,9 @@ def sink_prefill_mfma_supported(heads: int, kv_heads: int, dim: int, vdim: int, 
 
 def sink_attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
                            r1, r2, sink, talk, heads: int, kv_heads: int, dim: int, vdim: int, block_size: int, window: int,
-                           scale: float) -> None:
+                           scale: float, compute_units: int = 256) -> None:
     """``sink_attention`` on the matrix cores for bfloat16 portions: ``items`` are runs of up to
-    16 tokens. Scores, softmax and the mixing across heads are float32; the mixed weights meet
+    16 tokens; a launch of fewer runs than ``compute_units`` gives each run two workgroups. Scores, softmax and the mixing across heads are float32; the mixed weights meet
     the values as two bfloat16 operands (leading bits and rest)."""
     _gpu(q, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, r1, r2, sink, talk)
     T = q.shape[0]
@@ -1540,4 +1540,4 @@ def sink_attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables
     _check(_load("sink_attention").cw_sink_prefill_mfma(
         _ptr(q), q_stride, _ptr(out), _ptr(k_cache), _ptr(v_cache), rows, _ptr(block_tables), block_tables.shape[1],
         _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(r1), _ptr(r2), _ptr(sink), _ptr(talk), heads, kv_heads, dim,
-        vdim, block_size, int(window), float(scale), _stream()), "sink_attention_prefill")
+        vdim, block_size, int(window), float(scale), int(compute_units), _stream()), "sink_attention_prefill")

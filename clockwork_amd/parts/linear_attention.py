@@ -5,7 +5,7 @@ One product makes q, k, v, the output gate and the low-rank input of the decay f
 of the step; one kernel walks each request's tokens in order from the request's state slot
 (float32 [heads, key_dim, value_dim], zero at a request's start), makes the decays
 (sigmoid(z)^(1/tau) through log-sigmoid, float32), norms and gates the outputs; output product.
-A step with a portion of more than 64 tokens cuts every request's tokens into segments of 64 that
+A step with a portion of more than 64 tokens cuts every request's tokens into segments of 32 that
 are walked side by side: each from a zero state, then the start states are carried from segment
 to segment, then each segment is walked again for its outputs (the same sums, other parentheses).
 The state is all the mixer keeps: a ``StateSpec``.
@@ -23,7 +23,7 @@ from clockwork_amd.parts.specs import DecayedLinearAttentionSpec
 
 
 # tokens of a segment, and the longest portion that is still walked token by token in one piece
-SEGMENT_TOKENS = 64
+SEGMENT_TOKENS = 32
 SEGMENT_MIN_TOKENS = 64
 
 

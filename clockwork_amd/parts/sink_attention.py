@@ -138,7 +138,7 @@ class SinkAttention(Part):
                    cache.block_size, s.window or 0, s.scale)
         if n_items and self.mfma_ok:
             ops.sink_attention_prefill(qkv, qkv.shape[1], out, k_plane, v_plane, ctx.block_tables[cache.group], ctx.ctx_lens,
-                                       ctx.cu_q, items, n_items, *options)
+                                       ctx.cu_q, items, n_items, *options, compute_units=ctx.num_compute_units)
         elif n_items:
             ops.sink_attention(qkv, qkv.shape[1], out, k_plane, v_plane, ctx.block_tables[cache.group], ctx.ctx_lens,
                                ctx.cu_q, items, n_items, self.run, *options)

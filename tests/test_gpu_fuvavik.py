@@ -153,7 +153,7 @@ def test_gelu_feed_forward_and_the_capped_head(dtype):
     close(got.double().cpu(), want, dtype)
 
 
-def _step_through(part, need, x, cuts, dtype, block_size=8, num_blocks=16, release=True):
+def _step_through(part, need, x, cuts, dtype, block_size=8, num_blocks=16, release=True, compute_units=None):
     """Run ``x`` [T, hidden] through a mixer in steps of ``cuts`` tokens with a cache manager and
     NaN-poisoned pools of its own; returns the outputs, concatenated."""
     from clockwork_amd.cache import CacheManager, plan_groups
@@ -170,6 +170,8 @@ def _step_through(part, need, x, cuts, dtype, block_size=8, num_blocks=16, relea
             manager.admit("s", n)
         manager.extend("s", at, at + n)
         ctx = build_context([StepEntry("s", at, [0] * n)], manager, torch.device(DEV), 10)
+        if compute_units is not None:
+            ctx.num_compute_units = compute_units  # what the parts size their launches by
         if pools.state:
             pools.set_fresh_states(ctx.state_slots, ctx.starts, ctx.num_requests)
         got.append(part.forward(x[at : at + n].to(dtype).to(DEV), ctx, cache))
@@ -225,6 +227,9 @@ def test_sink_attention_whole_in_portions_and_token_by_token(dtype, shape):
         # alone, a tenth of what separates either from the float64 result
         assert dtype == torch.bfloat16
         fast = _step_through(part, part.cache_need(), x, [T], dtype)
+        # on a card of one compute unit a run's value columns are not shared between two workgroups
+        whole = _step_through(part, part.cache_need(), x, [T], dtype, compute_units=1)
+        assert float((fast - whole).abs().max()) < 1e-6 * max(1.0, float(fast.abs().max()))
         part.mfma_ok = False
         slow = _step_through(part, part.cache_need(), x, [T], dtype)
         scale = float(want.square().mean().sqrt())
