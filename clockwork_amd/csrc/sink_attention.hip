@@ -35,6 +35,7 @@ struct SinkAttnParams {
   float scale;
   int bq;                 // query tokens a workgroup takes at most
   int64_t cache_rows;
+  int tb_len;             // matrix-core kernel: entries of the block table a workgroup keeps in LDS
 };
 
 template <typename T>
@@ -240,7 +241,7 @@ CW_EXPORT int cw_sink_attention(int dtype, const void* q, int64_t q_stride, void
   p.block_tables = block_tables; p.table_width = table_width; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
   p.r1 = r1; p.r2 = r2; p.sink = sink; p.talk = talk;
   p.heads = heads; p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.block_size = block_size; p.window = window;
-  p.scale = scale; p.bq = bq; p.cache_rows = cache_rows;
+  p.scale = scale; p.bq = bq; p.cache_rows = cache_rows; p.tb_len = 0;
   const size_t smem = (size_t)sink_attention_lds_floats(bq, heads, dim, vdim) * sizeof(float);
   dim3 grid(n_items), block(256);
 #define CW_LAUNCH(T_)                                                                                             \
@@ -628,12 +629,17 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
   bf16_t* Vt = Ks + G * SM_KT * KROW;                            // [G][VW][VROW]
   float* Pn = reinterpret_cast<float*>(Vt + G * VW * VROW);      // [H][16][SM_PROW]
   float* Tk = Pn + H * 16 * SM_PROW;                             // [H][H]
+  int* Tb = reinterpret_cast<int*>(Tk + H * H);                  // [tb_len] pages of the keys this run sees
 
   const bf16_t* q = (const bf16_t*)p.q;
   const bf16_t* kc = (const bf16_t*)p.k_cache;
   const bf16_t* vc = (const bf16_t*)p.v_cache;
   if (p.talk)
     for (int i = tid; i < H * H; i += 256) Tk[i] = p.talk[i];
+  // the pages of the keys in [lo, last]: looked up once, so a chunk's loads do not wait for the table
+  const int tb0 = lo / p.block_size;
+  for (int i = tid; i < p.tb_len; i += 256) Tb[i] = tb0 + i < p.table_width ? table[tb0 + i] : -1;
+  __syncthreads();
 
   // this wave's heads and their query fragments: lane = query l16, 8 elements at slot
   sa_bf16x8_t qf[HPW][D32];
@@ -645,38 +651,70 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
     for (int ks = 0; ks < D32; ++ks) qf[a][ks] = sm_load8(q + (row0 + qi) * p.q_stride + g * D + ks * 32 + slot * 8);
   }
 
-  // the chunk's keys of every key/value head into LDS; keys past ``last`` or without a page: zeros
-  auto load_keys = [&](int k0) {
+  // A chunk's keys (and values) of every key/value head travel in two steps: from the pages into
+  // registers (asked for one chunk ahead, so the trip to memory runs beside the products of the
+  // chunk before), then into LDS. Keys past ``last`` or without a page are zeros. A thread moves up
+  // to PF pieces of 16 bytes of each (the host sees to it that this is enough).
+  constexpr int PF = 4;
+  uint4 kreg[PF], vreg[PF];
+  auto row_of = [&](int j) -> int64_t {
+    if (j > last) return -1;
+    const int slot_ = j / p.block_size - tb0;
+    const int page = slot_ < p.tb_len ? Tb[slot_] : -1;
+    const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
+    return page >= 0 && row < p.cache_rows ? row : -1;
+  };
+  auto fetch_keys = [&](int k0) {
     constexpr int PER_ROW = D / 8;
-    for (int idx = tid; idx < G * SM_KT * PER_ROW; idx += 256) {
-      const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
-      const int j = k0 + jj;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (j <= last) {
-        const int page = table[j / p.block_size];
-        const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
-        if (page >= 0 && row < p.cache_rows) v = *reinterpret_cast<const uint4*>(kc + (row * G + c) * D + e * 8);
+#pragma unroll
+    for (int it = 0; it < PF; ++it) {
+      const int idx = tid + it * 256;
+      kreg[it] = make_uint4(0, 0, 0, 0);
+      if (idx < G * SM_KT * PER_ROW) {
+        const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
+        const int64_t row = row_of(k0 + jj);
+        if (row >= 0) kreg[it] = *reinterpret_cast<const uint4*>(kc + (row * G + c) * D + e * 8);
       }
-      *reinterpret_cast<uint4*>(Ks + (c * SM_KT + jj) * KROW + e * 8) = v;
     }
   };
-  auto load_values = [&](int k0) {
-    constexpr int PER_ROW = VW / 8;
-    for (int idx = tid; idx < G * SM_KT * PER_ROW; idx += 256) {
-      const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
-      const int j = k0 + jj;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (j <= last) {
-        const int page = table[j / p.block_size];
-        const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
-        if (page >= 0 && row < p.cache_rows) v = *reinterpret_cast<const uint4*>(vc + (row * G + c) * V + v0 + e * 8);
-      }
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-      uint16_t* dst = reinterpret_cast<uint16_t*>(Vt) + (c * VW + e * 8) * VROW + jj;
+  auto store_keys = [&]() {
+    constexpr int PER_ROW = D / 8;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        dst[(2 * u) * VROW] = (uint16_t)(w[u] & 0xffffu);
-        dst[(2 * u + 1) * VROW] = (uint16_t)(w[u] >> 16);
+    for (int it = 0; it < PF; ++it) {
+      const int idx = tid + it * 256;
+      if (idx < G * SM_KT * PER_ROW) {
+        const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
+        *reinterpret_cast<uint4*>(Ks + (c * SM_KT + jj) * KROW + e * 8) = kreg[it];
+      }
+    }
+  };
+  auto fetch_values = [&](int k0) {
+    constexpr int PER_ROW = VW / 8;
+#pragma unroll
+    for (int it = 0; it < PF; ++it) {
+      const int idx = tid + it * 256;
+      vreg[it] = make_uint4(0, 0, 0, 0);
+      if (idx < G * SM_KT * PER_ROW) {
+        const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
+        const int64_t row = row_of(k0 + jj);
+        if (row >= 0) vreg[it] = *reinterpret_cast<const uint4*>(vc + (row * G + c) * V + v0 + e * 8);
+      }
+    }
+  };
+  auto store_values = [&]() {  // transposed: [dv][key]
+    constexpr int PER_ROW = VW / 8;
+#pragma unroll
+    for (int it = 0; it < PF; ++it) {
+      const int idx = tid + it * 256;
+      if (idx < G * SM_KT * PER_ROW) {
+        const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
+        const uint32_t w[4] = {vreg[it].x, vreg[it].y, vreg[it].z, vreg[it].w};
+        uint16_t* dst = reinterpret_cast<uint16_t*>(Vt) + (c * VW + e * 8) * VROW + jj;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          dst[(2 * u) * VROW] = (uint16_t)(w[u] & 0xffffu);
+          dst[(2 * u + 1) * VROW] = (uint16_t)(w[u] >> 16);
+        }
       }
     }
   };
@@ -712,9 +750,11 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
       l[a][e] = (p.sink && l16 == 0) ? 1.0f : 0.0f;
     }
   }
+  fetch_keys(lo);
   for (int k0 = lo; k0 <= last; k0 += SM_KT) {
     __syncthreads();
-    load_keys(k0);
+    store_keys();
+    if (k0 + SM_KT <= last) fetch_keys(k0 + SM_KT);
     __syncthreads();
 #pragma unroll
     for (int a = 0; a < HPW; ++a) {
@@ -754,10 +794,16 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
   for (int a = 0; a < HPW; ++a)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) out[a][nt] = sa_f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  fetch_keys(lo);
+  fetch_values(lo);
   for (int k0 = lo; k0 <= last; k0 += SM_KT) {
     __syncthreads();
-    load_keys(k0);
-    load_values(k0);
+    store_keys();
+    store_values();
+    if (k0 + SM_KT <= last) {
+      fetch_keys(k0 + SM_KT);
+      fetch_values(k0 + SM_KT);
+    }
     __syncthreads();
 #pragma unroll
     for (int a = 0; a < HPW; ++a) {
@@ -832,13 +878,16 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
 static int64_t sink_prefill_mfma_lds_bytes(int H, int G, int D, int V) {  // V: the value columns of one workgroup
   return (int64_t)G * SM_KT * (D + 8) * 2 + (int64_t)G * V * (SM_KT + 8) * 2 + (int64_t)H * 16 * SM_PROW * 4 + (int64_t)H * H * 4;
 }
+#define SM_MAX_TABLE 4096  // entries of the block table a workgroup keeps in LDS at most
 
 // The geometries this kernel is built for: dim 64 or 128, vdim 64 or 128, up to 16 heads
 // (4 a wave), and what of LDS they need.
 CW_EXPORT int cw_sink_prefill_mfma_supported(int heads, int kv_heads, int dim, int vdim) {
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || heads > 16) return 0;
   if ((dim != 64 && dim != 128) || (vdim != 64 && vdim != 128)) return 0;
-  return sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim) <= 150 * 1024 ? 1 : 0;
+  // a thread moves up to four 16-byte pieces of a chunk's keys, and of its values
+  if (kv_heads * SM_KT * (dim / 8) > 4 * 256 || kv_heads * SM_KT * (vdim / 8) > 4 * 256) return 0;
+  return sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim) + SM_MAX_TABLE * 4 <= 150 * 1024 ? 1 : 0;
 }
 
 // items: runs of up to 16 tokens. bfloat16 only. A launch of fewer than v_split_below runs gives
@@ -861,7 +910,12 @@ CW_EXPORT int cw_sink_prefill_mfma(const void* q, int64_t q_stride, void* out, c
   p.scale = scale; p.bq = 16; p.cache_rows = cache_rows;
   // few runs: two workgroups a run, each with half of the value columns
   const int vs = n_items < v_split_below ? 2 : 1;
-  const size_t smem = (size_t)sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim / vs);
+  // the pages a run of 16 tokens can see: its window and itself, or the whole table
+  int64_t tb_len = window > 0 ? (int64_t)(window + 16) / block_size + 2 : table_width;
+  if (tb_len > table_width) tb_len = table_width;
+  if (tb_len > SM_MAX_TABLE) return CW_ERR_SIZE;
+  p.tb_len = (int)tb_len;
+  const size_t smem = (size_t)sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim / vs) + (size_t)tb_len * 4;
   const dim3 grid(n_items, vs), block(256);
   const int hpw = (heads + 3) / 4;
 #define CW_LAUNCH_VS(HPW_, D32_, V16_, VS_)                                                                           \
