@@ -493,15 +493,15 @@ def measure_decode_attention_grid() -> dict:
 
 
 # Layer sizes for ``--design fuvavik``: widths, head counts and feed-forwards of the Qwen2.5
-# 0.5B / 1.5B / 7B layers, a window of half the prompt, a recurrence of as many heads with a
-# 64 x 128 state each. Beside each the Qwen2 layer of equal width, heads and feed-forward runs.
+# 0.5B / 1.5B / 3B layers, a window of half the prompt, a recurrence of as many heads with a
+# 64 x 64 or 64 x 128 state each. Beside each the Qwen2 layer of equal width, heads and feed-forward runs.
 FUVAVIK_SIZES = {
     "s": dict(width=896, heads=14, kv_heads=2, dim=64, vdim=64, window=1024, r_heads=14, r_dim=64, r_vdim=64, rank=16,
               ff=4864, layers=4),
     "m": dict(width=1536, heads=12, kv_heads=2, dim=128, vdim=128, window=1024, r_heads=12, r_dim=64, r_vdim=128, rank=32,
               ff=8960, layers=4),
-    "l": dict(width=3584, heads=28, kv_heads=4, dim=128, vdim=128, window=1024, r_heads=28, r_dim=64, r_vdim=128, rank=64,
-              ff=18944, layers=2),
+    "l": dict(width=2048, heads=16, kv_heads=2, dim=128, vdim=128, window=1024, r_heads=16, r_dim=64, r_vdim=128, rank=32,
+              ff=11008, layers=4),
 }
 DESIGN_VOCAB = 32768
 

@@ -360,15 +360,24 @@ __global__ __launch_bounds__(256) void sink_decode_scores_kernel(SinkDecodeParam
       for (int e = 0; e < SD_HG; ++e) acc[e] = 0.0f;
       if (there) {
         if (vec) {
-          for (int d = 0; d < D; d += N) {
-            float kv[N];
-            RowVec<T>::load(krow + d, kv);
+          // four pieces of the row are asked for together: a trip to memory that waits for the one
+          // before costs more than all the arithmetic of the row
+          for (int d0 = 0; d0 < D; d0 += 4 * N) {
+            float kv[4][N];
 #pragma unroll
-            for (int e = 0; e < SD_HG; ++e) {
-              if (h0 + e < Hg) {
-                const float* qv = qs + (c * Hg + h0 + e) * D + d;
+            for (int b = 0; b < 4; ++b)
+              if (d0 + b * N < D) RowVec<T>::load(krow + d0 + b * N, kv[b]);
 #pragma unroll
-                for (int u = 0; u < N; ++u) acc[e] += qv[u] * kv[u];
+            for (int b = 0; b < 4; ++b) {
+              if (d0 + b * N < D) {
+#pragma unroll
+                for (int e = 0; e < SD_HG; ++e) {
+                  if (h0 + e < Hg) {
+                    const float* qv = qs + (c * Hg + h0 + e) * D + d0 + b * N;
+#pragma unroll
+                    for (int u = 0; u < N; ++u) acc[e] += qv[u] * kv[b][u];
+                  }
+                }
               }
             }
           }
@@ -429,6 +438,9 @@ __global__ __launch_bounds__(256) void sink_decode_values_kernel(SinkDecodeParam
   float* mg = Pm + H * SK;       // [H] maxima
   float* il = mg + H;            // [H] 1 / denominators
   int* rows = (int*)(il + H);    // [SK] cache rows of the run's keys (-1: none)
+  float* tk = (float*)(rows + SK);  // [H][H] the mixing matrix
+  if (p.talk)
+    for (int i = tid; i < H * H; i += 256) tk[i] = p.talk[i];
   // every head's final maximum and denominator from the runs' own: a wave per head, a lane per run
   for (int g = tid >> 6; g < H; g += 4) {
     const int ln = tid & 63;
@@ -468,7 +480,7 @@ __global__ __launch_bounds__(256) void sink_decode_values_kernel(SinkDecodeParam
     for (int idx = tid; idx < H * SK; idx += 256) {
       const int h = idx / SK, jj = idx - h * SK;
       float v = 0.0f;
-      for (int g = 0; g < H; ++g) v += p.talk[h * H + g] * Pn[g * SK + jj];
+      for (int g = 0; g < H; ++g) v += tk[h * H + g] * Pn[g * SK + jj];
       Pm[idx] = v;
     }
     __syncthreads();
@@ -483,13 +495,22 @@ __global__ __launch_bounds__(256) void sink_decode_values_kernel(SinkDecodeParam
       float acc[SD_HG];
 #pragma unroll
       for (int e = 0; e < SD_HG; ++e) acc[e] = 0.0f;
-#pragma unroll 4
-      for (int jj = 0; jj < nk; ++jj) {
-        const int row = rows[jj];
-        const float v = row >= 0 ? cw_to_float(vc[((int64_t)row * G + c) * V + dv]) : 0.0f;
+      // thirty-two keys' values are asked for together: the trips to memory run side by side
+      for (int j0 = 0; j0 < nk; j0 += 32) {
+        float v[32];
 #pragma unroll
-        for (int e = 0; e < SD_HG; ++e)
-          if (h0 + e < Hg) acc[e] += W[(c * Hg + h0 + e) * SK + jj] * v;
+        for (int u = 0; u < 32; ++u) {
+          const int row = j0 + u < nk ? rows[j0 + u] : -1;
+          v[u] = row >= 0 ? cw_to_float(vc[((int64_t)row * G + c) * V + dv]) : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+          if (j0 + u < nk) {
+#pragma unroll
+            for (int e = 0; e < SD_HG; ++e)
+              if (h0 + e < Hg) acc[e] += W[(c * Hg + h0 + e) * SK + j0 + u] * v[u];
+          }
+        }
       }
 #pragma unroll
       for (int e = 0; e < SD_HG; ++e)
@@ -523,7 +544,7 @@ CW_EXPORT int64_t cw_sink_decode_workspace_floats(int n_requests, int n_runs, in
 CW_EXPORT int cw_sink_decode_supported(int heads, int kv_heads, int dim, int vdim) {
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return 0;
   const int64_t a = ((int64_t)heads * dim + (int64_t)heads * SD_MAX_SK) * 4;
-  const int64_t b = (2 * (int64_t)heads * SD_MAX_SK + 2 * heads + SD_MAX_SK) * 4;
+  const int64_t b = (2 * (int64_t)heads * SD_MAX_SK + 2 * heads + SD_MAX_SK + (int64_t)heads * heads) * 4;
   return a <= 150 * 1024 && b <= 150 * 1024 ? 1 : 0;
 }
 
@@ -552,7 +573,7 @@ CW_EXPORT int cw_sink_decode(int dtype, const void* q, int64_t q_stride, void* o
   p.heads = heads; p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.block_size = block_size; p.window = window;
   p.sk = sk; p.n_runs = n_runs; p.scale = scale; p.cache_rows = cache_rows;
   const size_t smem1 = ((size_t)heads * dim + (size_t)heads * sk) * sizeof(float);
-  const size_t smem2 = (2 * (size_t)heads * sk + 2 * heads + sk) * sizeof(float);
+  const size_t smem2 = (2 * (size_t)heads * sk + 2 * heads + sk + (size_t)heads * heads) * sizeof(float);
   const dim3 grid(n_requests, n_runs), block(256);
   int my = (heads * vdim + 255) / 256;
   if (my > 64) my = 64;
