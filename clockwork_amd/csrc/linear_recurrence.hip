@@ -224,6 +224,7 @@ struct SegParams {
   void* out;
   int heads, dim, vdim, rank, n_slots, n_tokens;
   float q_scale, inv_tau, eps;
+  int seg_tokens;         // the most tokens a segment has
 };
 
 template <typename T> struct LrVec;
@@ -280,9 +281,10 @@ __global__ __launch_bounds__(256) void lrs_prepare_kernel(SegParams p) {
 // MODE 0: from zero, leaves ``added`` and ``seg_decay``; MODE 1: from the start state in ``added``
 // (the carry kernel has turned it into that), writes the raw outputs.
 template <typename T, int DIM, int MODE>
-__global__ __launch_bounds__(64) void lrs_walk_kernel(SegParams p) {
+__global__ __launch_bounds__(256) void lrs_walk_kernel(SegParams p) {
+  extern __shared__ __align__(16) float tile[];  // the segment's decays, keys and queries: [3][tokens][D]
   const int seg = blockIdx.x, h = blockIdx.y;
-  const int v = blockIdx.z * 64 + threadIdx.x;
+  const int v = blockIdx.z * blockDim.x + threadIdx.x;
   const int r = p.seg_items[4 * seg], tok0 = p.seg_items[4 * seg + 1], ntok = p.seg_items[4 * seg + 2];
   const int q_len = p.cu_q[r + 1] - p.cu_q[r];
   const int slot = p.state_slots[r];
@@ -307,12 +309,25 @@ __global__ __launch_bounds__(64) void lrs_walk_kernel(SegParams p) {
     for (int d = 0; d < DIM; ++d) A[d] = 1.0f;
   }
   const T* proj = (const T*)p.proj;
+  // the waves of the workgroup (each 64 columns of the same head's state) share the segment's
+  // decays, keys and queries through LDS: fetched once, in whole rows, then read by every lane at
+  // the same address (a broadcast) while the tokens are walked
+  float* As = tile;
+  float* Kt = As + p.seg_tokens * D;
+  float* Qt = Kt + p.seg_tokens * D;
+  for (int i = threadIdx.x; i < nt * D; i += blockDim.x) {
+    const int t = i / D, d = i - t * D;
+    const int64_t at = (row0 + t) * HD + h * D + d;
+    As[i] = p.dec[at];
+    Kt[i] = p.kf[at];
+    if (MODE == 1) Qt[i] = p.qf[at];
+  }
+  __syncthreads();
   for (int t = 0; t < nt; ++t) {
     const int64_t row = row0 + t;
-    // the same addresses in every lane: scalar loads
-    const float* a = p.dec + row * HD + h * D;
-    const float* k = p.kf + row * HD + h * D;
-    const float* q = p.qf + row * HD + h * D;
+    const float* a = As + t * D;
+    const float* k = Kt + t * D;
+    const float* q = Qt + t * D;
     const float vv = cw_to_float(proj[row * p.stride + p.v_off + h * V + vc]);
     float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
 #pragma unroll
@@ -410,7 +425,7 @@ CW_EXPORT int64_t cw_linear_recurrence_segments_workspace_floats(int n_tokens, i
 CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t stride, int q_off, int k_off, int v_off,
                                             int g_off, int u_off, const void* a2, const float* a2b, const float* norm_w,
                                             float* state, int n_slots, const int* state_slots, const int* cu_q,
-                                            const int* seg_items, int n_segments, const int* req_first, float* workspace,
+                                            const int* seg_items, int n_segments, int seg_tokens, const int* req_first, float* workspace,
                                             void* out, int n_requests, int n_tokens, int heads, int dim, int vdim, int rank,
                                             float q_scale, float inv_tau, float eps, hipStream_t stream) {
   if (n_requests < 0 || n_tokens < 0 || n_segments < 0 || !proj || !a2 || !state || !state_slots || !cu_q || !seg_items ||
@@ -422,6 +437,7 @@ CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t
     return CW_ERR_ARG;
   if (!cw_linear_recurrence_segments_supported(dim, vdim)) return CW_ERR_SIZE;
   if (heads > 65535 || (vdim + 63) / 64 > 65535) return CW_ERR_SIZE;
+  if (seg_tokens < 1 || (int64_t)3 * seg_tokens * dim * 4 > 48 * 1024) return CW_ERR_SIZE;
   if (n_requests == 0 || n_tokens == 0 || n_segments == 0) return CW_OK;
   SegParams p;
   p.proj = proj; p.stride = stride; p.q_off = q_off; p.k_off = k_off; p.v_off = v_off; p.g_off = g_off; p.u_off = u_off;
@@ -436,14 +452,17 @@ CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t
   p.raw = p.seg_decay + (int64_t)n_segments * heads * dim;
   int64_t pb = (THD + 255) / 256;
   if (pb > 65536) pb = 65536;
-  const dim3 walk_grid(n_segments, heads, (vdim + 63) / 64);
+  p.seg_tokens = seg_tokens;
+  const int walk_threads = vdim >= 256 ? 256 : 64 * ((vdim + 63) / 64);   // up to four waves share a segment's rows
+  const dim3 walk_grid(n_segments, heads, (vdim + walk_threads - 1) / walk_threads);
+  const size_t walk_lds = (size_t)3 * seg_tokens * dim * sizeof(float);
   const dim3 carry_grid(n_requests, heads, (unsigned)(((int64_t)dim * vdim + 255) / 256));
   const unsigned finish_blocks = (unsigned)(((int64_t)n_tokens * heads + 3) / 4);
 #define CW_WALK(T_, DIM_)                                                                          \
   do {                                                                                             \
-    hipLaunchKernelGGL((lrs_walk_kernel<T_, DIM_, 0>), walk_grid, dim3(64), 0, stream, p);         \
+    hipLaunchKernelGGL((lrs_walk_kernel<T_, DIM_, 0>), walk_grid, dim3(walk_threads), walk_lds, stream, p); \
     hipLaunchKernelGGL(lrs_carry_kernel, carry_grid, dim3(256), 0, stream, p);                     \
-    hipLaunchKernelGGL((lrs_walk_kernel<T_, DIM_, 1>), walk_grid, dim3(64), 0, stream, p);         \
+    hipLaunchKernelGGL((lrs_walk_kernel<T_, DIM_, 1>), walk_grid, dim3(walk_threads), walk_lds, stream, p); \
   } while (0)
 #define CW_ALL(T_)                                                                                 \
   do {                                                                                             \

@@ -141,7 +141,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_linear_recurrence": [I, P, L, I, I, I, I, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, F, F, P],
             "cw_linear_recurrence_segments_supported": [I, I],
             "cw_linear_recurrence_segments_workspace_floats": [I, I, I, I, I],
-            "cw_linear_recurrence_segments": [I, P, L, I, I, I, I, I, P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, I, I,
+            "cw_linear_recurrence_segments": [I, P, L, I, I, I, I, I, P, P, P, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I,
                                               F, F, F, P],
         },
         "sampling": {
@@ -1438,13 +1438,14 @@ def linear_recurrence_segments_supported(dim: int, vdim: int) -> bool:
 
 
 def linear_recurrence_segments(proj, q_off: int, k_off: int, v_off: int, g_off: int, u_off: int, a2, a2_bias, norm_weight,
-                               state, state_slots, cu_q, seg_items, n_segments: int, req_first, n_requests: int, heads: int,
-                               dim: int, vdim: int, q_scale: float, tau: float, eps: float) -> torch.Tensor:
+                               state, state_slots, cu_q, seg_items, n_segments: int, seg_tokens: int, req_first,
+                               n_requests: int, heads: int, dim: int, vdim: int, q_scale: float, tau: float,
+                               eps: float) -> torch.Tensor:
     """``linear_recurrence`` for steps with long portions: the tokens are cut into segments that
     are walked side by side (each from a zero state, then the segments' start states are carried
     from the request's slot, then each is walked again for its outputs). ``seg_items`` int32
     [n_segments, 4]: (request, first token of the segment in the request's portion, tokens, 0),
-    a request's segments in order and together; ``req_first`` int32 [R + 1]: where each
+    a request's segments in order and together, none longer than ``seg_tokens``; ``req_first`` int32 [R + 1]: where each
     request's segments begin. The same arguments and result otherwise."""
     _gpu(proj, a2, a2_bias, norm_weight, state, state_slots, cu_q, seg_items, req_first)
     T, width = proj.shape
@@ -1463,7 +1464,7 @@ def linear_recurrence_segments(proj, q_off: int, k_off: int, v_off: int, g_off: 
     _check(lib.cw_linear_recurrence_segments(
         dtype_code(proj.dtype), _ptr(proj), width, q_off, k_off, v_off, g_off, u_off, _ptr(a2), _ptr(a2_bias),
         _ptr(norm_weight), _ptr(state), state.shape[0], _ptr(state_slots), _ptr(cu_q), _ptr(seg_items), n_segments,
-        _ptr(req_first), _ptr(workspace), _ptr(out), n_requests, T, heads, dim, vdim, a2.shape[1], float(q_scale),
+        int(seg_tokens), _ptr(req_first), _ptr(workspace), _ptr(out), n_requests, T, heads, dim, vdim, a2.shape[1], float(q_scale),
         1.0 / float(tau), float(eps), _stream()), "linear_recurrence_segments")
     return out
 

@@ -105,7 +105,7 @@ class DecayedLinearAttention(Part):
         plan = self._segments(ctx)
         if plan is not None:
             items, n_segments, first = plan
-            out = ops.linear_recurrence_segments(*common, items, n_segments, first, *sizes)
+            out = ops.linear_recurrence_segments(*common, items, n_segments, SEGMENT_TOKENS, first, *sizes)
         else:
             out = ops.linear_recurrence(*common, *sizes)
         return ops.linear(out, self.out_weight, policy=policy)
