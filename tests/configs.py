@@ -121,5 +121,18 @@ FUVAVIK_C = {
     "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
     "layers": [_fuvavik_layer(1, 1, 32, 8, 0.18, 17, 1, 16, 4, 8.0, 1, 24)],
 }
+# four layers of unlike sizes for long requests: windows of 77 to 1500, key and value sizes that the
+# matrix-core attention kernel takes (layers 1 to 3) and one that it does not, states from 16 x 16 to
+# 128 x 256
+FUVAVIK_LONG = {
+    "architecture": "Fuvavik", "vocab": 211, "width": 192, "max_positions": 1600,
+    "embedding": {"scale": 1.7}, "norm": {"eps": 2e-6}, "logit_softcap": 11.0,
+    "layers": [
+        _fuvavik_layer(6, 3, 32, 48, 0.3, 200, 3, 40, 24, 8.0, 12, 384),
+        _fuvavik_layer(4, 4, 64, 64, 0.2, 77, 2, 64, 128, 32.0, 8, None),
+        _fuvavik_layer(8, 2, 128, 64, 0.15, 513, 6, 16, 16, 2.0, 4, 100),
+        _fuvavik_layer(16, 2, 64, 128, 0.2, 1500, 1, 128, 256, 64.0, 16, 64),
+    ],
+}
 # name -> (config, weight seed, cache block size)
 FUVAVIK_CONFIGS = {"FA": (FUVAVIK_A, 21, 8), "FB": (FUVAVIK_B, 22, 16), "FC": (FUVAVIK_C, 23, 4)}

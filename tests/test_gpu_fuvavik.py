@@ -455,6 +455,28 @@ def test_models_in_four_batching_modes(fuvavik_dirs, name, mode, dtype):
     assert all(p.num_free == runner.manager.num_blocks for p in runner.manager.pools)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_requests_through_layers_of_unlike_sizes(tmp_path, dtype):
+    """1400 and 333 tokens through four layers that share no size: windows of 77 to 1500 pass over
+    hundreds of tokens, keys far back are inside the longest and outside the others, the
+    matrix-core kernel serves three of the four layers in bfloat16, the recurrence runs in
+    segments; whole, prefill then single tokens, portions of 2 to 512 tokens, and mixed."""
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests.configs import FUVAVIK_LONG
+
+    model_dir = write_random_model(tmp_path / "long", FUVAVIK_LONG, 5)
+    requests = _requests(211, [1400, 333], seed=3)
+    oracle = plain.PlainFuvavik(model_dir)
+    ref = {rid: oracle.logits(toks) for rid, toks in requests.items()}
+    for mode in ("whole", "prefill_then_decode", "portions", "mixed"):
+        runner = replay.make_runner(model_dir, dtype, 16, 120, max_model_len=1600)
+        if dtype == "bfloat16":
+            assert [m.left.mfma_ok for m in runner.model.mixers()] == [False, True, True, True]
+        steps = replay.portions(requests, sizes=[2, 300, 7, 64, 129, 33, 512]) if mode == "portions" else getattr(replay, mode)(requests)
+        _check(replay.run_trace(runner, steps), ref, dtype)
+        assert all(p.num_free == runner.manager.num_blocks for p in runner.manager.pools)
+
+
 def test_cache_groups_of_a_model_whose_layers_differ(fuvavik_dirs):
     runner = replay.make_runner(fuvavik_dirs["FB"], "float32", 16, 40)
     groups = [(g.is_kv, g.window, g.entries) for g in runner.manager.groups]
