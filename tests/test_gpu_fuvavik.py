@@ -199,6 +199,7 @@ LEFT_SHAPES = [
     (3, 1, 40, 24, 300, 50),
     (1, 1, 8, 72, 1, 40),
     (16, 4, 64, 32, 20, 96),
+    (5, 5, 20, 12, 11, 40),   # rows that are no multiple of 16 bytes: the kernels' element-by-element loads
     # the sizes that the matrix-core kernel for bfloat16 portions takes
     (12, 2, 128, 128, 40, 64),
     (6, 3, 64, 128, 23, 48),
@@ -303,6 +304,46 @@ def test_one_loud_key_just_inside_and_just_outside_the_window(window, cuts):
         steps = {"whole": [T], "portions": [2, 7, 3, 16, 5, 2, 31, 4], "single": [loud + 2] + [1] * (T - loud - 2)}[cuts]
         got = _step_through(part, part.cache_need(), x, steps, torch.float32, block_size=block_size, num_blocks=24)
         torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_far_key_among_hundreds_decides_the_output(dtype):
+    """The same loud key behind a window of 400: it is one of up to 400 keys that a query sees, 399
+    positions back at the last one that sees it, and gone at the next. In bfloat16 the portions
+    run on the matrix cores and the single tokens share their keys among several workgroups."""
+    hidden, heads, dim, vdim, window = 32, 2, 64, 64, 400
+    spec = SinkAttentionSpec(hidden_size=hidden, num_heads=heads, num_kv_heads=1, key_dim=dim, value_dim=vdim, scale=1.0,
+                             window=window, qk_norm_eps=1e-6, distance_bias=False, talking_heads=False)
+    part = build_part(spec)
+
+    def change(v):
+        v["qkv_weight"].zero_()
+        v["qkv_weight"][0, 1] = 1.0
+        v["qkv_weight"][dim, 1] = 1.0
+        v["qkv_weight"][2 * dim, 0] = 1.0
+        v["qkv_weight"][2 * dim + 1, 1] = 0.05
+        v["qkv_weight"][3 * dim, 0] = 1.0
+        v["q_norm"].fill_(6.0)
+        v["k_norm"].fill_(6.0)
+        v["sink"].fill_(-2.0)
+        v["out_weight"].zero_()
+        v["out_weight"][0, 0] = 1.0
+        v["out_weight"][1, vdim] = 1.0
+
+    w = bind(part, dtype, change=change)
+    assert part.mfma_ok == (dtype == torch.bfloat16)
+    T, loud = 450, 7
+    x = torch.zeros(T, hidden)
+    x[:, 1] = 1.0
+    x[loud, 0] = 4.0
+    names = _left_names({**w, "r1": torch.zeros(2, dtype=torch.float64), "r2": torch.zeros(2, dtype=torch.float64),
+                         "talk": torch.eye(2, dtype=torch.float64)}, spec)
+    want = plain.sink_window_attention(x.double(), names, "", _left_sizes(spec), 1e-6)
+    assert float(want[loud + window - 1, 0]) > 3.9 and abs(float(want[loud + window, 0])) < 1e-6
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    for steps in ([T], [2, 300, 7, 64, 29, 33, 15], [390] + [1] * 60):
+        got = _step_through(part, part.cache_need(), x, steps, dtype, block_size=16, num_blocks=40)
+        torch.testing.assert_close(got, want, **tol)
 
 
 def _right_names(w, spec):
