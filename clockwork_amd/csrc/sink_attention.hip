@@ -342,34 +342,40 @@ __global__ __launch_bounds__(256) void sink_decode_scores_kernel(SinkDecodeParam
   const T* kc = (const T*)p.k_cache;
   constexpr int N = RowVec<T>::N;
   const bool vec = D % N == 0 && !((uintptr_t)kc & 15);
-  for (int idx = tid; idx < SK * G; idx += 256) {
+  // a run of few keys leaves threads over: 2, 4 or 8 neighbouring lanes then share a key's row
+  // (each a run of its elements) and add their sums up with shuffles
+  int tpk = 1;
+  while (vec && tpk < 8 && SK * G * tpk * 2 <= 256 && D % (tpk * 2 * N) == 0) tpk *= 2;
+  const int dpt = D / tpk;  // elements of a row that a thread takes
+  for (int idx0 = tid; idx0 < SK * G * tpk; idx0 += 256) {
+    const int idx = idx0 / tpk, piece = idx0 - idx * tpk;
     const int c = idx / SK, jj = idx - c * SK;
     const int j = k0 + jj;
     const bool seen = j <= pos;
-    const T* krow = kc;
-    bool there = false;
-    if (seen) {
-      const int page = table[j / p.block_size];
-      const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
-      there = page >= 0 && row < p.cache_rows;
-      if (there) krow = kc + (row * G + c) * D;
-    }
+    // a key that is not seen or has no page reads row 0 and its products are dropped: every
+    // thread's loads are then the same instructions, asked for together
+    const int jt = min(j, pos);
+    const int page = table[jt / p.block_size];
+    const int64_t row = (int64_t)page * p.block_size + jt % p.block_size;
+    const bool there = seen && page >= 0 && row < p.cache_rows;
+    const T* krow = kc + ((there ? row : 0) * G + c) * D;
     for (int h0 = 0; h0 < Hg; h0 += SD_HG) {
       float acc[SD_HG];
 #pragma unroll
       for (int e = 0; e < SD_HG; ++e) acc[e] = 0.0f;
-      if (there) {
+      {
         if (vec) {
           // four pieces of the row are asked for together: a trip to memory that waits for the one
           // before costs more than all the arithmetic of the row
-          for (int d0 = 0; d0 < D; d0 += 4 * N) {
+          const int d_end = (piece + 1) * dpt;
+          for (int d0 = piece * dpt; d0 < d_end; d0 += 4 * N) {
             float kv[4][N];
 #pragma unroll
             for (int b = 0; b < 4; ++b)
-              if (d0 + b * N < D) RowVec<T>::load(krow + d0 + b * N, kv[b]);
+              if (d0 + b * N < d_end) RowVec<T>::load(krow + d0 + b * N, kv[b]);
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
-              if (d0 + b * N < D) {
+              if (d0 + b * N < d_end) {
 #pragma unroll
                 for (int e = 0; e < SD_HG; ++e) {
                   if (h0 + e < Hg) {
@@ -382,7 +388,7 @@ __global__ __launch_bounds__(256) void sink_decode_scores_kernel(SinkDecodeParam
             }
           }
         } else {
-          for (int d = 0; d < D; ++d) {
+          for (int d = piece * dpt; d < (piece + 1) * dpt; ++d) {
             const float kv = cw_to_float(krow[d]);
 #pragma unroll
             for (int e = 0; e < SD_HG; ++e)
@@ -390,11 +396,15 @@ __global__ __launch_bounds__(256) void sink_decode_scores_kernel(SinkDecodeParam
           }
         }
       }
+      for (int off = 1; off < tpk; off <<= 1) {
+#pragma unroll
+        for (int e = 0; e < SD_HG; ++e) acc[e] += __shfl_xor(acc[e], off, 64);
+      }
 #pragma unroll
       for (int e = 0; e < SD_HG; ++e) {
-        if (h0 + e < Hg) {
+        if (h0 + e < Hg && piece == 0) {
           const int g = c * Hg + h0 + e;
-          float s = acc[e] * p.scale;
+          float s = there ? acc[e] * p.scale : 0.0f;
           if (p.r1) s -= p.r1[g] * log1pf(p.r2[g] * (float)max(pos - j, 0));
           sc[g * SK + jj] = seen ? s : -INFINITY;
         }
@@ -500,8 +510,11 @@ __global__ __launch_bounds__(256) void sink_decode_values_kernel(SinkDecodeParam
         float v[32];
 #pragma unroll
         for (int u = 0; u < 32; ++u) {
+          // the load itself is unconditional (row 0 stands in, its value is dropped): a load under a
+          // condition of its own is waited for before the next one is asked for
           const int row = j0 + u < nk ? rows[j0 + u] : -1;
-          v[u] = row >= 0 ? cw_to_float(vc[((int64_t)row * G + c) * V + dv]) : 0.0f;
+          const float x = cw_to_float(vc[((int64_t)max(row, 0) * G + c) * V + dv]);
+          v[u] = row >= 0 ? x : 0.0f;
         }
 #pragma unroll
         for (int u = 0; u < 32; ++u) {
@@ -679,23 +692,23 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
   constexpr int PF = 4;
   uint4 kreg[PF], vreg[PF];
   auto row_of = [&](int j) -> int64_t {
-    if (j > last) return -1;
-    const int slot_ = j / p.block_size - tb0;
-    const int page = slot_ < p.tb_len ? Tb[slot_] : -1;
+    const int slot_ = min(max(j / p.block_size - tb0, 0), p.tb_len - 1);
+    const int page = Tb[slot_];
     const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
-    return page >= 0 && row < p.cache_rows ? row : -1;
+    return (j <= last && j / p.block_size - tb0 < p.tb_len && page >= 0 && row < p.cache_rows) ? row : -1;
   };
   auto fetch_keys = [&](int k0) {
     constexpr int PER_ROW = D / 8;
 #pragma unroll
     for (int it = 0; it < PF; ++it) {
       const int idx = tid + it * 256;
-      kreg[it] = make_uint4(0, 0, 0, 0);
-      if (idx < G * SM_KT * PER_ROW) {
-        const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
-        const int64_t row = row_of(k0 + jj);
-        if (row >= 0) kreg[it] = *reinterpret_cast<const uint4*>(kc + (row * G + c) * D + e * 8);
-      }
+      // every load is unconditional (a piece past the chunk or without a page reads row 0 and is
+      // dropped): loads under conditions of their own would be waited for one by one
+      const int at = min(idx, G * SM_KT * PER_ROW - 1);
+      const int e = at % PER_ROW, jj = (at / PER_ROW) % SM_KT, c = at / (PER_ROW * SM_KT);
+      const int64_t row = row_of(k0 + jj);
+      const uint4 x = *reinterpret_cast<const uint4*>(kc + ((row >= 0 ? row : 0) * G + c) * D + e * 8);
+      kreg[it] = (row >= 0 && idx == at) ? x : make_uint4(0, 0, 0, 0);
     }
   };
   auto store_keys = [&]() {
@@ -714,12 +727,11 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
 #pragma unroll
     for (int it = 0; it < PF; ++it) {
       const int idx = tid + it * 256;
-      vreg[it] = make_uint4(0, 0, 0, 0);
-      if (idx < G * SM_KT * PER_ROW) {
-        const int e = idx % PER_ROW, jj = (idx / PER_ROW) % SM_KT, c = idx / (PER_ROW * SM_KT);
-        const int64_t row = row_of(k0 + jj);
-        if (row >= 0) vreg[it] = *reinterpret_cast<const uint4*>(vc + (row * G + c) * V + v0 + e * 8);
-      }
+      const int at = min(idx, G * SM_KT * PER_ROW - 1);
+      const int e = at % PER_ROW, jj = (at / PER_ROW) % SM_KT, c = at / (PER_ROW * SM_KT);
+      const int64_t row = row_of(k0 + jj);
+      const uint4 x = *reinterpret_cast<const uint4*>(vc + ((row >= 0 ? row : 0) * G + c) * V + v0 + e * 8);
+      vreg[it] = (row >= 0 && idx == at) ? x : make_uint4(0, 0, 0, 0);
     }
   };
   auto store_values = [&]() {  // transposed: [dv][key]
