@@ -81,14 +81,14 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnParams p) {
   auto load_rows = [&](const T* cache, int width, int c, int k0, float* dst, int dst_stride) {
     for (int idx = tid; idx < SA_KT * width; idx += 256) {
       const int jj = idx / width, e = idx - jj * width;
-      const int j = k0 + jj;
-      float v = 0.0f;
-      if (j <= last) {
-        const int page = table[j / p.block_size];
-        const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
-        if (page >= 0 && row < p.cache_rows) v = cw_to_float(cache[(row * G + c) * width + e]);
-      }
-      dst[jj * dst_stride + e] = v;
+      // the loads are unconditional (a key past ``last`` or without a page reads row 0 and is dropped
+      // by a select): loads under conditions of their own would be waited for one by one
+      const int j = min(k0 + jj, last);
+      const int page = table[j / p.block_size];
+      const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
+      const bool there = k0 + jj <= last && page >= 0 && row < p.cache_rows;
+      const float v = cw_to_float(cache[((there ? row : 0) * G + c) * width + e]);
+      dst[jj * dst_stride + e] = there ? v : 0.0f;
     }
   };
   const int lane = tid % SA_LANES, rgroup = tid / SA_LANES;  // 16 groups of 16 lanes
