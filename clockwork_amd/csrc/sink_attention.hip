@@ -751,25 +751,45 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
       }
     }
   };
-  // the scores of head g's tile kt of the chunk: rows slot * 4 + e, key 16 kt + l16; -inf where not seen
-  auto scores = [&](int a, int g, int kt, int k0, float* s) {
+  // the scores of head g against the chunk's 32 keys, in units of log 2 (so that the softmax takes
+  // bare exp2 instructions): s[kt * 4 + e] is row slot * 4 + e, key 16 kt + l16; -inf where not
+  // seen. The two tiles' products are issued in turn. ``inside``: every pair of the chunk is seen
+  // (most chunks of a long window), so nothing is tested.
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float scale2 = p.scale * LOG2E;
+  auto scores = [&](int a, int g, int k0, bool inside, float* s) {
     const int c = g / Hg;
-    sa_f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
-    const bf16_t* kb = Ks + (c * SM_KT + kt * 16 + l16) * KROW + slot * 8;
+    sa_f32x4_t acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bf16_t* kb = Ks + (c * SM_KT + l16) * KROW + slot * 8;
 #pragma unroll
-    for (int ks = 0; ks < D32; ++ks)
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[a][ks], sm_load8(kb + ks * 32), acc, 0, 0, 0);
-    const int j = k0 + kt * 16 + l16;
+    for (int ks = 0; ks < D32; ++ks) {
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[a][ks], sm_load8(kb + ks * 32), acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[a][ks], sm_load8(kb + 16 * KROW + ks * 32), acc1, 0, 0, 0);
+    }
+    // r1 * ln(1 + r2 d) in units of log 2 is r1 * log2(1 + r2 d)
     const float r1 = p.r1 ? p.r1[g] : 0.0f, r2 = p.r1 ? p.r2[g] : 0.0f;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int i = slot * 4 + e;
-      const int dist = pos0 + i - j;
-      float v = acc[e] * p.scale;
-      if (p.r1) v -= r1 * __logf(1.0f + r2 * (float)max(dist, 0));
-      const bool seen = i < nq && dist >= 0 && (p.window <= 0 || dist < p.window);
-      s[e] = seen ? v : -INFINITY;
+    for (int kt = 0; kt < 2; ++kt) {
+      const int j = k0 + kt * 16 + l16;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = slot * 4 + e;
+        const int dist = pos0 + i - j;
+        float v = (kt == 0 ? acc0[e] : acc1[e]) * scale2;
+        if (inside) {
+          if (p.r1) v -= r1 * __builtin_amdgcn_logf(1.0f + r2 * (float)dist);
+          s[kt * 4 + e] = v;
+        } else {
+          if (p.r1) v -= r1 * __builtin_amdgcn_logf(1.0f + r2 * (float)max(dist, 0));
+          const bool seen = i < nq && dist >= 0 && (p.window <= 0 || dist < p.window);
+          s[kt * 4 + e] = seen ? v : -INFINITY;
+        }
+      }
     }
+  };
+  // is every pair of (one of the run's 16 rows, one of the chunk's 32 keys) seen?
+  auto all_seen = [&](int k0) {
+    return nq == 16 && k0 + SM_KT - 1 <= pos0 && (p.window <= 0 || pos0 + 15 - k0 < p.window);
   };
 
   // ---- first walk: maxima and denominators, per lane, then across the 16 lanes of a row
@@ -779,7 +799,7 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
     const int g = min(wave + 4 * a, H - 1);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      m[a][e] = p.sink ? p.sink[g] : -3.0e38f;
+      m[a][e] = p.sink ? p.sink[g] * LOG2E : -3.0e38f;
       l[a][e] = (p.sink && l16 == 0) ? 1.0f : 0.0f;
     }
   }
@@ -789,20 +809,19 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
     store_keys();
     if (k0 + SM_KT <= last) fetch_keys(k0 + SM_KT);
     __syncthreads();
+    const bool inside = all_seen(k0);
 #pragma unroll
     for (int a = 0; a < HPW; ++a) {
       const int g = wave + 4 * a;
       if (g < H) {
+        float s[8];
+        scores(a, g, k0, inside, s);
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-          float s[4];
-          scores(a, g, kt, k0, s);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float mn = fmaxf(m[a][e], s[e]);
-            l[a][e] = l[a][e] * __expf(m[a][e] - mn) + __expf(s[e] - mn);
-            m[a][e] = mn;
-          }
+        for (int e = 0; e < 4; ++e) {
+          const float mn = fmaxf(m[a][e], fmaxf(s[e], s[4 + e]));
+          l[a][e] = l[a][e] * __builtin_amdgcn_exp2f(m[a][e] - mn) + __builtin_amdgcn_exp2f(s[e] - mn) +
+                    __builtin_amdgcn_exp2f(s[4 + e] - mn);
+          m[a][e] = mn;
         }
       }
     }
@@ -815,7 +834,7 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
       for (int off = 8; off > 0; off >>= 1) {
         const float mo = __shfl_xor(m[a][e], off, 16), lo_ = __shfl_xor(l[a][e], off, 16);
         const float mn = fmaxf(m[a][e], mo);
-        l[a][e] = l[a][e] * __expf(m[a][e] - mn) + lo_ * __expf(mo - mn);
+        l[a][e] = l[a][e] * __builtin_amdgcn_exp2f(m[a][e] - mn) + lo_ * __builtin_amdgcn_exp2f(mo - mn);
         m[a][e] = mn;
       }
       l[a][e] = l[a][e] > 0.0f ? 1.0f / l[a][e] : 0.0f;  // from here on: 1 / denominator
@@ -838,18 +857,19 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
       fetch_values(k0 + SM_KT);
     }
     __syncthreads();
+    const bool inside = all_seen(k0);
 #pragma unroll
     for (int a = 0; a < HPW; ++a) {
       const int g = wave + 4 * a;
       if (g < H) {
+        float s[8];
+        scores(a, g, k0, inside, s);
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-          float s[4];
-          scores(a, g, kt, k0, s);
+        for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            Pn[(g * 16 + slot * 4 + e) * SM_PROW + kt * 16 + l16] = __expf(s[e] - m[a][e]) * l[a][e];
-        }
+            Pn[(g * 16 + slot * 4 + e) * SM_PROW + kt * 16 + l16] =
+                __builtin_amdgcn_exp2f(s[kt * 4 + e] - m[a][e]) * l[a][e];
       }
     }
     __syncthreads();
