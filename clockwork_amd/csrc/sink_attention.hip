@@ -928,6 +928,260 @@ __global__ __launch_bounds__(256) void sink_prefill_mfma_kernel(SinkAttnParams p
   }
 }
 
+// ======================================================================================
+// The same portions in ONE walk over the keys, for models of one or two key/value heads. The
+// mixing across heads is linear: head h's output is
+//   sum over g of talk[h, g] / denominator(g) * (unnormalised weights of head g) . V of h's key/value head,
+// so a wave keeps, for each of its query heads, one accumulator per key/value head (with the
+// usual running maximum), and the finished, normalised accumulators are mixed once at the end,
+// through LDS. Scores are made as K Q^T: a lane then holds, for ITS query (l16), the chunk's keys
+// 4 slot + e and 16 + 4 slot + e, which is the A operand of the value product as it lies in the
+// registers (the value fragments are read with the keys in that order). Weights are float32 and
+// fed as two bfloat16 operands, as in the kernel above.
+// ======================================================================================
+template <int HPW, int D32, int V16, int VS, int GC>
+__global__ __launch_bounds__(256) void sink_prefill_onewalk_kernel(SinkAttnParams p) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  constexpr int D = D32 * 32, V = V16 * 16, NT = V16 / VS, VW = NT * 16;
+  const int v0 = blockIdx.y * VW;
+  constexpr int KROW = D + 8;
+  constexpr int VROW = SM_KT + 8;
+  const int H = p.heads, G = GC, Hg = H / G;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l16 = lane & 15, slot = lane >> 4;
+  const int r = p.items[4 * blockIdx.x], tok0 = p.items[4 * blockIdx.x + 1];
+  const int q_len = p.cu_q[r + 1] - p.cu_q[r];
+  if (tok0 >= q_len) return;
+  const int nq = min(min(p.items[4 * blockIdx.x + 2], 16), q_len - tok0);
+  const int pos0 = p.ctx_lens[r] - q_len + tok0;
+  const int last = pos0 + nq - 1;
+  const int lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
+  const int64_t row0 = p.cu_q[r] + tok0;
+  const int* table = p.block_tables + (int64_t)r * p.table_width;
+
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(smem_raw);              // [G][KT][KROW]
+  bf16_t* Vt = Ks + G * SM_KT * KROW;                            // [G][VW][VROW]
+  float* Ox = reinterpret_cast<float*>(smem_raw);                // at the end, over the tiles: [H][16][VW] finished outputs of one key/value head
+  const int tile_bytes = (G * SM_KT * KROW + G * VW * VROW) * 2, finish_bytes = H * 16 * VW * 4;
+  float* Tk = reinterpret_cast<float*>(smem_raw + max(tile_bytes, finish_bytes));  // [H][H], behind both
+  int* Tb = reinterpret_cast<int*>(Tk + H * H);                  // [tb_len]
+
+  const bf16_t* q = (const bf16_t*)p.q;
+  const bf16_t* kc = (const bf16_t*)p.k_cache;
+  const bf16_t* vc = (const bf16_t*)p.v_cache;
+  for (int i = tid; i < H * H; i += 256) Tk[i] = p.talk ? p.talk[i] : (i / H == i % H ? 1.0f : 0.0f);
+  const int tb0 = lo / p.block_size;
+  for (int i = tid; i < p.tb_len; i += 256) Tb[i] = tb0 + i < p.table_width ? table[tb0 + i] : -1;
+  __syncthreads();
+
+  // query fragments as the B operand: lane = query l16, 8 elements at slot
+  sa_bf16x8_t qf[HPW][D32];
+  const int qi = min(l16, nq - 1);
+#pragma unroll
+  for (int a = 0; a < HPW; ++a) {
+    const int g = min(wave + 4 * a, H - 1);
+#pragma unroll
+    for (int ks = 0; ks < D32; ++ks) qf[a][ks] = sm_load8(q + (row0 + qi) * p.q_stride + g * D + ks * 32 + slot * 8);
+  }
+
+  constexpr int PF = 4;
+  uint4 kreg[PF], vreg[PF];
+  auto row_of = [&](int j) -> int64_t {
+    const int slot_ = min(max(j / p.block_size - tb0, 0), p.tb_len - 1);
+    const int page = Tb[slot_];
+    const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
+    return (j <= last && j / p.block_size - tb0 < p.tb_len && page >= 0 && row < p.cache_rows) ? row : -1;
+  };
+  auto fetch = [&](int k0) {
+    constexpr int KPR = D / 8, VPR = VW / 8;
+#pragma unroll
+    for (int it = 0; it < PF; ++it) {
+      const int idx = tid + it * 256;
+      {
+        const int at = min(idx, G * SM_KT * KPR - 1);
+        const int e = at % KPR, jj = (at / KPR) % SM_KT, c = at / (KPR * SM_KT);
+        const int64_t row = row_of(k0 + jj);
+        const uint4 x = *reinterpret_cast<const uint4*>(kc + ((row >= 0 ? row : 0) * G + c) * D + e * 8);
+        kreg[it] = (row >= 0 && idx == at) ? x : make_uint4(0, 0, 0, 0);
+      }
+      {
+        const int at = min(idx, G * SM_KT * VPR - 1);
+        const int e = at % VPR, jj = (at / VPR) % SM_KT, c = at / (VPR * SM_KT);
+        const int64_t row = row_of(k0 + jj);
+        const uint4 x = *reinterpret_cast<const uint4*>(vc + ((row >= 0 ? row : 0) * G + c) * V + v0 + e * 8);
+        vreg[it] = (row >= 0 && idx == at) ? x : make_uint4(0, 0, 0, 0);
+      }
+    }
+  };
+  auto store = [&]() {
+    constexpr int KPR = D / 8, VPR = VW / 8;
+#pragma unroll
+    for (int it = 0; it < PF; ++it) {
+      const int idx = tid + it * 256;
+      if (idx < G * SM_KT * KPR) {
+        const int e = idx % KPR, jj = (idx / KPR) % SM_KT, c = idx / (KPR * SM_KT);
+        *reinterpret_cast<uint4*>(Ks + (c * SM_KT + jj) * KROW + e * 8) = kreg[it];
+      }
+      if (idx < G * SM_KT * VPR) {
+        const int e = idx % VPR, jj = (idx / VPR) % SM_KT, c = idx / (VPR * SM_KT);
+        const uint32_t w[4] = {vreg[it].x, vreg[it].y, vreg[it].z, vreg[it].w};
+        uint16_t* dst = reinterpret_cast<uint16_t*>(Vt) + (c * VW + e * 8) * VROW + jj;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          dst[(2 * u) * VROW] = (uint16_t)(w[u] & 0xffffu);
+          dst[(2 * u + 1) * VROW] = (uint16_t)(w[u] >> 16);
+        }
+      }
+    }
+  };
+
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float scale2 = p.scale * LOG2E;
+  // per head: the query's running maximum (the same in the 4 lanes of a query), this lane's part
+  // of its denominator, and the accumulators, one per key/value head
+  float m[HPW], l[HPW];
+  sa_f32x4_t out[HPW][GC][NT];
+#pragma unroll
+  for (int a = 0; a < HPW; ++a) {
+    const int g = min(wave + 4 * a, H - 1);
+    m[a] = p.sink ? p.sink[g] * LOG2E : -3.0e38f;
+    l[a] = (p.sink && slot == 0) ? 1.0f : 0.0f;
+#pragma unroll
+    for (int c = 0; c < GC; ++c)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) out[a][c][nt] = sa_f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+
+  fetch(lo);
+  for (int k0 = lo; k0 <= last; k0 += SM_KT) {
+    __syncthreads();
+    store();
+    if (k0 + SM_KT <= last) fetch(k0 + SM_KT);
+    __syncthreads();
+    const bool inside = nq == 16 && k0 + SM_KT - 1 <= pos0 && (p.window <= 0 || pos0 + 15 - k0 < p.window);
+    sa_bf16x8_t ph[HPW], pl[HPW];
+#pragma unroll
+    for (int a = 0; a < HPW; ++a) {
+      const int g = wave + 4 * a;
+      if (g < H) {
+        const int c = g / Hg;
+        // S^T tiles: rows = keys 16 kt + 4 slot + e, column = this lane's query
+        sa_f32x4_t acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+        const bf16_t* kb = Ks + (c * SM_KT + l16) * KROW + slot * 8;
+#pragma unroll
+        for (int ks = 0; ks < D32; ++ks) {
+          acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sm_load8(kb + ks * 32), qf[a][ks], acc0, 0, 0, 0);
+          acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sm_load8(kb + 16 * KROW + ks * 32), qf[a][ks], acc1, 0, 0, 0);
+        }
+        const float r1 = p.r1 ? p.r1[g] : 0.0f, r2 = p.r1 ? p.r2[g] : 0.0f;
+        float s[8];
+        float top = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int j = k0 + (u >> 2) * 16 + slot * 4 + (u & 3);
+          const int dist = pos0 + l16 - j;
+          float v = (u < 4 ? acc0[u & 3] : acc1[u & 3]) * scale2;
+          if (p.r1) v -= r1 * __builtin_amdgcn_logf(1.0f + r2 * (float)max(dist, 0));
+          if (!inside) {
+            const bool seen = l16 < nq && dist >= 0 && (p.window <= 0 || dist < p.window);
+            v = seen ? v : -INFINITY;
+          }
+          s[u] = v;
+          top = fmaxf(top, v);
+        }
+        top = cw_quad_max(top);
+        const float mn = fmaxf(m[a], top);
+        const float alpha = __builtin_amdgcn_exp2f(m[a] - mn);
+        m[a] = mn;
+        float sum = 0.0f;
+        float w[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          w[u] = __builtin_amdgcn_exp2f(s[u] - mn);
+          sum += w[u];
+        }
+        l[a] = l[a] * alpha + sum;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const __bf16 t = (__bf16)w[u];
+          ph[a][u] = t;
+          pl[a][u] = (__bf16)(w[u] - (float)t);
+        }
+        // the accumulators' rows are queries slot * 4 + e: each takes its own query's factor
+        if (__ballot(alpha != 1.0f) != 0) {
+          float ar[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) ar[e] = __shfl(alpha, slot * 4 + e, 64);
+#pragma unroll
+          for (int cc = 0; cc < GC; ++cc)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) out[a][cc][nt][e] *= ar[e];
+        }
+      }
+    }
+    // values: a fragment (one key/value head, 16 value columns) serves all of the wave's heads
+#pragma unroll
+    for (int cc = 0; cc < GC; ++cc) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        // column l16 of the tile, keys 4 slot .. + 4 and 16 + 4 slot .. + 4: the order the weights lie in
+        const bf16_t* vb = Vt + (cc * VW + nt * 16 + l16) * VROW + slot * 4;
+        const uint2 lo4 = *reinterpret_cast<const uint2*>(vb), hi4 = *reinterpret_cast<const uint2*>(vb + 16);
+        const uint4 both = make_uint4(lo4.x, lo4.y, hi4.x, hi4.y);
+        const sa_bf16x8_t vf = *reinterpret_cast<const sa_bf16x8_t*>(&both);
+#pragma unroll
+        for (int a = 0; a < HPW; ++a) {
+          if (wave + 4 * a < H) {
+            out[a][cc][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph[a], vf, out[a][cc][nt], 0, 0, 0);
+            out[a][cc][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl[a], vf, out[a][cc][nt], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- finish: denominators, then the mixing across heads, one key/value head at a time through LDS
+  float inv_row[HPW][4];
+#pragma unroll
+  for (int a = 0; a < HPW; ++a) {
+    const float total = cw_quad_sum(l[a]);
+    const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) inv_row[a][e] = __shfl(inv, slot * 4 + e, 64);
+  }
+  bf16_t* o = (bf16_t*)p.out;
+  for (int cc = 0; cc < GC; ++cc) {
+    __syncthreads();  // the tiles (and the round before) are done with LDS
+#pragma unroll
+    for (int a = 0; a < HPW; ++a) {
+      const int g = wave + 4 * a;
+      if (g < H) {
+#pragma unroll
+        for (int c2 = 0; c2 < GC; ++c2) {
+          if (c2 == cc) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                Ox[(g * 16 + slot * 4 + e) * VW + nt * 16 + l16] = out[a][c2][nt][e] * inv_row[a][e];
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // heads of this key/value head: h = cc * Hg .. ; every thread takes outputs (h, query, column)
+    const int n_out = Hg * 16 * VW;
+    for (int idx = tid; idx < n_out; idx += 256) {
+      const int col = idx % VW, i = (idx / VW) % 16, h = cc * Hg + idx / (VW * 16);
+      float v = 0.0f;
+      for (int g = 0; g < H; ++g) v += Tk[h * H + g] * Ox[(g * 16 + i) * VW + col];
+      if (i < nq) o[(row0 + i) * (int64_t)(H * V) + h * V + v0 + col] = __float2bfloat16(v);
+    }
+  }
+}
+
 static int64_t sink_prefill_mfma_lds_bytes(int H, int G, int D, int V) {  // V: the value columns of one workgroup
   return (int64_t)G * SM_KT * (D + 8) * 2 + (int64_t)G * V * (SM_KT + 8) * 2 + (int64_t)H * 16 * SM_PROW * 4 + (int64_t)H * H * 4;
 }
@@ -941,6 +1195,12 @@ CW_EXPORT int cw_sink_prefill_mfma_supported(int heads, int kv_heads, int dim, i
   // a thread moves up to four 16-byte pieces of a chunk's keys, and of its values
   if (kv_heads * SM_KT * (dim / 8) > 4 * 256 || kv_heads * SM_KT * (vdim / 8) > 4 * 256) return 0;
   return sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim) + SM_MAX_TABLE * 4 <= 150 * 1024 ? 1 : 0;
+}
+
+static int64_t sink_prefill_onewalk_lds_bytes(int H, int G, int D, int VW) {  // without the pages' table
+  const int64_t tiles = (int64_t)G * SM_KT * (D + 8) * 2 + (int64_t)G * VW * (SM_KT + 8) * 2;
+  const int64_t finish = (int64_t)H * 16 * VW * 4;   // laid over the tiles; the mixing matrix and the pages lie behind both
+  return (tiles > finish ? tiles : finish) + (int64_t)H * H * 4;
 }
 
 // items: runs of up to 16 tokens. bfloat16 only. A launch of fewer than v_split_below runs gives
@@ -968,9 +1228,42 @@ CW_EXPORT int cw_sink_prefill_mfma(const void* q, int64_t q_stride, void* out, c
   if (tb_len > table_width) tb_len = table_width;
   if (tb_len > SM_MAX_TABLE) return CW_ERR_SIZE;
   p.tb_len = (int)tb_len;
-  const size_t smem = (size_t)sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim / vs) + (size_t)tb_len * 4;
   const dim3 grid(n_items, vs), block(256);
   const int hpw = (heads + 3) / 4;
+  // one or two key/value heads: the kernel that walks the keys once (two workgroups a run always:
+  // its accumulators for all value columns would not fit the registers)
+  if (kv_heads <= 2 && sink_prefill_onewalk_lds_bytes(heads, kv_heads, dim, vdim / 2) + tb_len * 4 <= 150 * 1024) {
+    const size_t smem1 = (size_t)sink_prefill_onewalk_lds_bytes(heads, kv_heads, dim, vdim / 2) + (size_t)tb_len * 4;
+    const dim3 grid1(n_items, 2);
+#define CW_ONE(HPW_, D32_, V16_, GC_)                                                                                 \
+  do {                                                                                                                \
+    if (smem1 > 48 * 1024 && hipFuncSetAttribute((const void*)sink_prefill_onewalk_kernel<HPW_, D32_, V16_, 2, GC_>,  \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess) \
+      return CW_ERR_LAUNCH;                                                                                           \
+    hipLaunchKernelGGL((sink_prefill_onewalk_kernel<HPW_, D32_, V16_, 2, GC_>), grid1, block, smem1, stream, p);      \
+  } while (0)
+#define CW_ONE_HEADS(D32_, V16_, GC_)              \
+  do {                                             \
+    if (hpw <= 1) CW_ONE(1, D32_, V16_, GC_);      \
+    else if (hpw == 2) CW_ONE(2, D32_, V16_, GC_); \
+    else if (hpw == 3) CW_ONE(3, D32_, V16_, GC_); \
+    else CW_ONE(4, D32_, V16_, GC_);               \
+  } while (0)
+#define CW_ONE_SIZES(GC_)                                        \
+  do {                                                           \
+    if (dim == 64 && vdim == 64) CW_ONE_HEADS(2, 4, GC_);        \
+    else if (dim == 64 && vdim == 128) CW_ONE_HEADS(2, 8, GC_);  \
+    else if (dim == 128 && vdim == 64) CW_ONE_HEADS(4, 4, GC_);  \
+    else CW_ONE_HEADS(4, 8, GC_);                                \
+  } while (0)
+    if (kv_heads == 1) CW_ONE_SIZES(1);
+    else CW_ONE_SIZES(2);
+#undef CW_ONE_SIZES
+#undef CW_ONE_HEADS
+#undef CW_ONE
+    return cw_launch_status();
+  }
+  const size_t smem = (size_t)sink_prefill_mfma_lds_bytes(heads, kv_heads, dim, vdim / vs) + (size_t)tb_len * 4;
 #define CW_LAUNCH_VS(HPW_, D32_, V16_, VS_)                                                                           \
   do {                                                                                                                \
     if (smem > 48 * 1024 && hipFuncSetAttribute((const void*)sink_prefill_mfma_kernel<HPW_, D32_, V16_, VS_>,         \
