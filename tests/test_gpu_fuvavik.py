@@ -205,6 +205,9 @@ LEFT_SHAPES = [
     (6, 3, 64, 128, 23, 48),
     (16, 16, 128, 64, 300, 32),
     (1, 1, 64, 64, 7, 40),
+    (14, 2, 64, 64, 50, 56),    # heads that the four waves do not share evenly
+    (6, 2, 128, 64, 19, 48),
+    (8, 4, 64, 64, 30, 64),     # more than two key/value heads: the keys are walked twice
 ]
 
 
