@@ -52,6 +52,16 @@ class GroupLayout:
     def window(self) -> Optional[int]:
         return self.need.window if self.is_kv else None
 
+    @property
+    def segment(self) -> Optional[int]:
+        """Positions a segment holds when tokens read the earlier tokens of their own segment only."""
+        return getattr(self.need, "segment", None) if self.is_kv else None
+
+    @property
+    def keeps_all(self) -> bool:
+        """Does a request keep every page of the group until it ends?"""
+        return self.window is None and self.segment is None
+
 
 def plan_groups(needs: Sequence[Optional[object]]) -> list[GroupLayout]:
     """``needs[i]`` is what run entry ``i`` stores (None: nothing of its own).
@@ -122,7 +132,7 @@ class CacheManager:
     def supports_prefix_sharing(self) -> bool:
         """Cached pages are a function of the token prefix alone only when every group keeps
         all keys and nothing else is carried from token to token."""
-        return bool(self.kv_groups) and not self.state_groups and all(g.window is None for g in self.kv_groups)
+        return bool(self.kv_groups) and not self.state_groups and all(g.keeps_all for g in self.kv_groups)
 
     def _next_epoch(self) -> int:
         self._epochs += 1
@@ -154,7 +164,10 @@ class CacheManager:
 
     def _first_needed_block(self, g: int, computed: int) -> int:
         """Logical block of the oldest key the token at position ``computed`` reads in group g."""
-        window = self.kv_groups[g].window
+        group = self.kv_groups[g]
+        if group.segment is not None:
+            return (computed // group.segment) * group.segment // self.block_size
+        window = group.window
         if window is None:
             return 0
         return max(0, computed - window + 1) // self.block_size
@@ -163,7 +176,7 @@ class CacheManager:
     def _admission_extent(self, g: int, total_len: int, portion_end: int) -> int:
         # a full group reserves the whole request up front (the reference's arithmetic,
         # block_manager.py:25-40); a windowed group only what the first portion touches
-        return total_len if self.kv_groups[g].window is None else portion_end
+        return total_len if self.kv_groups[g].keeps_all else portion_end
 
     def can_admit(self, total_len: int, portion_end: Optional[int] = None,
                   prefix_blocks: int = 0) -> bool:
@@ -287,7 +300,7 @@ class CacheManager:
         rec = self._requests[seq_id]
         given_back = 0
         for g, pool in enumerate(self.pools):
-            if self.kv_groups[g].window is None:
+            if self.kv_groups[g].keeps_all:
                 continue
             first = min(self._first_needed_block(g, computed), len(rec.tables[g]))
             for b in range(rec.released[g], first):

@@ -65,11 +65,14 @@ class PagedRowsSpec:
     and sharing work as for :class:`KVPagesSpec` (which is the case of two equal planes named
     ``k`` and ``v``); the mixer finds its planes in ``EntryCache.planes`` by name, each a flat
     [num_blocks * block_size, *row shape] view, and addresses them through the step's block
-    tables and slots of its group.
+    tables and slots of its group. ``segment`` S (instead of a window): positions are cut into
+    segments of S counted from 0 and a token reads the earlier tokens of its own segment only;
+    pages wholly before the segment of the next token are given back while the request runs.
     """
 
     planes: tuple
     window: Optional[int] = None
+    segment: Optional[int] = None
 
     def __post_init__(self):
         names = [name for name, _ in self.planes]
@@ -78,9 +81,14 @@ class PagedRowsSpec:
         for name, shape in self.planes:
             if not shape or any(int(d) < 1 for d in shape):
                 raise ValueError(f"plane {name!r} has no valid row shape: {shape!r}")
+        if self.window is not None and self.segment is not None:
+            raise ValueError("a paged cache has a window or segments, not both")
+        if self.segment is not None and self.segment < 1:
+            raise ValueError(f"segment must be positive, got {self.segment}")
 
     def group_key(self) -> tuple:
-        return ("rows", tuple((name, tuple(shape)) for name, shape in self.planes), self.window)
+        key = ("rows", tuple((name, tuple(shape)) for name, shape in self.planes), self.window)
+        return key if self.segment is None else key + (("segment", self.segment),)
 
 
 @dataclass(frozen=True)
@@ -158,11 +166,15 @@ class RunEntry:
 
     A layer may appear in several entries (its weights are then shared; each
     entry still has a cache of its own). ``cache_from`` names an *earlier entry*
-    whose cache this entry reads instead of writing its own.
+    whose cache this entry reads instead of writing its own. ``add_input``: the model's input
+    (what the embedding part made of the step's tokens) is added to the residual stream once
+    more right before this entry's block (a repeated run of layers that is fed the input again
+    at every pass); the block's first norm must be able to add it (``accepts_stream_input``).
     """
 
     layer: int
     cache_from: Optional[int] = None
+    add_input: bool = False
 
 
 @dataclass

@@ -1,8 +1,10 @@
 // Row-wise kernels of blocks other than the pre-norm RMSNorm / SwiGLU one, for gfx950:
 // embedding with a scale and a learned position table, residual add + LayerNorm (weight and
 // bias), the sigmoid-gated residual add of two branches, act(gate) * up for the tanh form of GELU,
-// the logit cap, the mean of two RMS-normed rows, and the RMS norm of whole query / key
-// projections fused with the cache write.
+// the logit cap, the mean of two RMS-normed rows, the RMS norm of whole query / key
+// projections fused with the cache write, residual add + Dynamic Tanh, the erf GELU, a sigmoid
+// gate, biased projections into cache rows, the low-rank query step with the latent cache row,
+// and the rotation of one part of every head.
 // Statistics, gates and the residual stream are float32; T is the activation type.
 #include "common.h"
 
@@ -330,5 +332,259 @@ CW_EXPORT int cw_qk_rownorm_store(void* proj, int dtype, int64_t stride, int q_o
   else if (dtype == CW_BF16 && wt == CW_F32) CW_LAUNCH(bf16_t, float);
   else return CW_ERR_DTYPE;
 #undef CW_LAUNCH
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- residual add + Dynamic Tanh
+// resid[t, :] += scale * delta[t, :] (+ extra[t, :]), then out = tanh(alpha * resid) * w + b: a norm
+// that takes no statistics of the row. ``extra`` is a float32 stream that joins the sum after the
+// branch (the model's input, added again before a repeated run of layers). With ``rows`` only
+// those rows are produced and resid is left alone. alpha is one element on the device.
+template <typename DT, typename WT, typename OT>
+__global__ __launch_bounds__(256) void add_dyt_kernel(float* __restrict__ resid, const DT* __restrict__ delta, float scale,
+                                                      const float* __restrict__ extra, const WT* __restrict__ w,
+                                                      const WT* __restrict__ b, const float* __restrict__ alpha,
+                                                      OT* __restrict__ out, const int* __restrict__ rows, int H) {
+  const int64_t i = blockIdx.x;
+  const int64_t src = rows ? (int64_t)rows[i] : i;
+  const float a = alpha[0];
+  float* r = resid + src * H;
+  for (int j = threadIdx.x; j < H; j += 256) {
+    float x = r[j];
+    if (delta) x += scale * cw_to_float(delta[src * H + j]);
+    if (extra) x += extra[src * H + j];
+    if (!rows && (delta || extra)) r[j] = x;
+    float y = tanhf(a * x) * cw_to_float(w[j]);
+    if (b) y += cw_to_float(b[j]);
+    out[i * H + j] = cw_from_float<OT>(y);
+  }
+}
+
+CW_EXPORT int cw_add_dyt(float* resid, const void* delta, int delta_dtype, float scale, const float* extra, const void* w,
+                         const void* b, int w_dtype, const float* alpha, void* out, int out_dtype, const int* rows, int n,
+                         int H, hipStream_t stream) {
+  if (n < 0 || H <= 0 || !resid || !w || !alpha || !out) return CW_ERR_ARG;
+  if (n == 0) return CW_OK;
+  dim3 grid(n), block(256);
+#define CW_LAUNCH(DT_, WT_, OT_)                                                                                  \
+  hipLaunchKernelGGL((add_dyt_kernel<DT_, WT_, OT_>), grid, block, 0, stream, resid, (const DT_*)delta, scale, extra, \
+                     (const WT_*)w, (const WT_*)b, alpha, (OT_*)out, rows, H)
+  const int dd = delta ? delta_dtype : out_dtype;
+  if (dd == CW_F32 && w_dtype == CW_F32 && out_dtype == CW_F32) CW_LAUNCH(float, float, float);
+  else if (dd == CW_BF16 && w_dtype == CW_BF16 && out_dtype == CW_BF16) CW_LAUNCH(bf16_t, bf16_t, bf16_t);
+  else if (dd == CW_BF16 && w_dtype == CW_F32 && out_dtype == CW_BF16) CW_LAUNCH(bf16_t, float, bf16_t);
+  else return CW_ERR_DTYPE;
+#undef CW_LAUNCH
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- erf GELU, in place
+// x <- 0.5 x (1 + erf(x / sqrt 2)), float32 inside.
+template <typename T>
+__global__ void gelu_erf_kernel(T* __restrict__ x, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const float z = cw_to_float(x[i]);
+    x[i] = cw_from_float<T>(0.5f * z * (1.0f + erff(z * 0.70710678118654752440f)));
+  }
+}
+
+CW_EXPORT int cw_gelu_erf(void* x, int dtype, int64_t n, hipStream_t stream) {
+  if (n < 0) return CW_ERR_ARG;
+  if (n == 0) return CW_OK;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 262144) blocks = 262144;
+  dim3 grid((unsigned)blocks), block(256);
+  if (dtype == CW_F32) hipLaunchKernelGGL(gelu_erf_kernel<float>, grid, block, 0, stream, (float*)x, n);
+  else if (dtype == CW_BF16) hipLaunchKernelGGL(gelu_erf_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)x, n);
+  else return CW_ERR_DTYPE;
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- a * sigmoid(z), in place on a
+// a[t, j] <- a[t, j] / (1 + exp(-z[t, z_off + j])), j < n; z rows are z_stride elements apart.
+template <typename T>
+__global__ void sigmoid_mul_kernel(T* __restrict__ a, const T* __restrict__ z, int64_t z_stride, int z_off, int n,
+                                   int64_t total) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / n;
+    const int j = (int)(i % n);
+    const float g = 1.0f / (1.0f + expf(-cw_to_float(z[t * z_stride + z_off + j])));
+    a[i] = cw_from_float<T>(cw_to_float(a[i]) * g);
+  }
+}
+
+CW_EXPORT int cw_sigmoid_mul(void* a, const void* z, int dtype, int64_t z_stride, int z_off, int T, int n,
+                             hipStream_t stream) {
+  if (T < 0 || n <= 0 || z_off < 0 || z_off + n > z_stride) return CW_ERR_ARG;
+  if (T == 0) return CW_OK;
+  const int64_t total = (int64_t)T * n;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 262144) blocks = 262144;
+  dim3 grid((unsigned)blocks), block(256);
+  if (dtype == CW_F32)
+    hipLaunchKernelGGL(sigmoid_mul_kernel<float>, grid, block, 0, stream, (float*)a, (const float*)z, z_stride, z_off, n, total);
+  else if (dtype == CW_BF16)
+    hipLaunchKernelGGL(sigmoid_mul_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)a, (const bf16_t*)z, z_stride, z_off, n, total);
+  else return CW_ERR_DTYPE;
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- biases and the cache write, no positions
+// A row of proj holds a token's query, key and value projections at q_off / k_off / v_off. The
+// bias (one element per column of proj, or nullptr) is added: the queries are rewritten in place,
+// keys and values go to the rows k_plane[slot, nk] and v_plane[slot, nv]. A negative slot writes
+// no cache row.
+template <typename T, typename WT>
+__global__ __launch_bounds__(256) void bias_store_kernel(T* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off,
+                                                         int nq, int nk, int nv, const WT* __restrict__ bias,
+                                                         const int* __restrict__ slots, T* __restrict__ k_plane,
+                                                         T* __restrict__ v_plane, int64_t cache_rows) {
+  const int64_t t = blockIdx.x;
+  T* row = proj + t * stride;
+  int64_t slot = slots ? (int64_t)slots[t] : -1;
+  if (slot >= cache_rows) slot = -1;
+  if (bias)
+    for (int j = threadIdx.x; j < nq; j += 256)
+      row[q_off + j] = cw_from_float<T>(cw_to_float(row[q_off + j]) + cw_to_float(bias[q_off + j]));
+  if (slot >= 0) {
+    T* kd = k_plane + slot * nk;
+    for (int j = threadIdx.x; j < nk; j += 256)
+      kd[j] = cw_from_float<T>(cw_to_float(row[k_off + j]) + (bias ? cw_to_float(bias[k_off + j]) : 0.0f));
+    T* vd = v_plane + slot * nv;
+    for (int j = threadIdx.x; j < nv; j += 256)
+      vd[j] = cw_from_float<T>(cw_to_float(row[v_off + j]) + (bias ? cw_to_float(bias[v_off + j]) : 0.0f));
+  }
+}
+
+CW_EXPORT int cw_bias_store(void* proj, int dtype, int64_t stride, int q_off, int k_off, int v_off, int nq, int nk, int nv,
+                            const void* bias, int b_dtype, const int* slots, void* k_plane, void* v_plane,
+                            int64_t cache_rows, int T, hipStream_t stream) {
+  if (T < 0 || nq < 0 || nk < 0 || nv < 0 || q_off < 0 || k_off < 0 || v_off < 0) return CW_ERR_ARG;
+  if (q_off + nq > stride || k_off + nk > stride || v_off + nv > stride) return CW_ERR_ARG;
+  if (slots && (!k_plane || !v_plane)) return CW_ERR_ARG;
+  if (T == 0) return CW_OK;
+  dim3 grid(T), block(256);
+#define CW_LAUNCH(T_, WT_)                                                                                         \
+  hipLaunchKernelGGL((bias_store_kernel<T_, WT_>), grid, block, 0, stream, (T_*)proj, stride, q_off, k_off, v_off, nq, \
+                     nk, nv, (const WT_*)bias, slots, (T_*)k_plane, (T_*)v_plane, cache_rows)
+  const int wt = bias ? b_dtype : dtype;
+  if (dtype == CW_F32 && wt == CW_F32) CW_LAUNCH(float, float);
+  else if (dtype == CW_BF16 && wt == CW_BF16) CW_LAUNCH(bf16_t, bf16_t);
+  else if (dtype == CW_BF16 && wt == CW_F32) CW_LAUNCH(bf16_t, float);
+  else return CW_ERR_DTYPE;
+#undef CW_LAUNCH
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- low-rank queries and the latent cache row
+// A row of proj holds, at dq_off, nq elements of a query's low-rank step and, at dkv_off,
+// rank + rot elements of the key/value one. One workgroup a token:
+//   cq[t, :]            = dq / rms(dq) * wq                      (T, [T, nq])
+//   plane[slot, :rank]  = dkv[:rank] / rms(dkv[:rank]) * wkv     (the latent)
+//   plane[slot, rank:]  = dkv[rank:] with its first rdims elements rotated by the token's position:
+//                         pairs (i, i + rdims / 2), angle = float(position) * freq[i]
+// rms(x) = sqrt(mean(x^2) + eps), float32.
+template <typename T, typename WT>
+__global__ __launch_bounds__(256) void latent_store_kernel(const T* __restrict__ proj, int64_t stride, int dq_off, int nq,
+                                                           int dkv_off, int rank, int rot, int rdims,
+                                                           const WT* __restrict__ wq, const WT* __restrict__ wkv, float eps,
+                                                           const int* __restrict__ positions,
+                                                           const float* __restrict__ freq, const int* __restrict__ slots,
+                                                           T* __restrict__ cq, T* __restrict__ plane, int64_t cache_rows) {
+  __shared__ float scratch[4];
+  const int64_t t = blockIdx.x;
+  const T* row = proj + t * stride;
+  int64_t slot = slots ? (int64_t)slots[t] : -1;
+  if (slot >= cache_rows) slot = -1;
+  float sq = 0.0f, sk = 0.0f;
+  for (int j = threadIdx.x; j < nq; j += 256) { const float v = cw_to_float(row[dq_off + j]); sq += v * v; }
+  for (int j = threadIdx.x; j < rank; j += 256) { const float v = cw_to_float(row[dkv_off + j]); sk += v * v; }
+  const float iq = 1.0f / sqrtf(block_sum_256(sq, scratch) / (float)nq + eps);
+  const float ik = 1.0f / sqrtf(block_sum_256(sk, scratch) / (float)rank + eps);
+  for (int j = threadIdx.x; j < nq; j += 256)
+    cq[t * nq + j] = cw_from_float<T>(cw_to_float(row[dq_off + j]) * iq * cw_to_float(wq[j]));
+  if (slot < 0) return;
+  T* dst = plane + slot * (rank + rot);
+  for (int j = threadIdx.x; j < rank; j += 256)
+    dst[j] = cw_from_float<T>(cw_to_float(row[dkv_off + j]) * ik * cw_to_float(wkv[j]));
+  const float pos = (float)positions[t];
+  const int half = rdims / 2;
+  const T* r = row + dkv_off + rank;
+  for (int j = threadIdx.x; j < rot; j += 256) {
+    float v = cw_to_float(r[j]);
+    if (j < rdims) {
+      const int i = j < half ? j : j - half;
+      float s, c;
+      sincosf(pos * freq[i], &s, &c);
+      const float u = cw_to_float(r[i]), w = cw_to_float(r[i + half]);
+      v = j < half ? u * c - w * s : w * c + u * s;
+    }
+    dst[rank + j] = cw_from_float<T>(v);
+  }
+}
+
+CW_EXPORT int cw_latent_store(const void* proj, int dtype, int64_t stride, int dq_off, int nq, int dkv_off, int rank, int rot,
+                              int rdims, const void* wq, const void* wkv, int w_dtype, float eps, const int* positions,
+                              const float* freq, const int* slots, void* cq, void* plane, int64_t cache_rows, int T,
+                              hipStream_t stream) {
+  if (T < 0 || nq <= 0 || rank <= 0 || rot < 0 || rdims < 0 || rdims > rot || (rdims & 1)) return CW_ERR_ARG;
+  if (dq_off < 0 || dkv_off < 0 || dq_off + nq > stride || dkv_off + rank + rot > stride) return CW_ERR_ARG;
+  if (!proj || !wq || !wkv || !cq || !positions || (rdims && !freq) || (slots && !plane)) return CW_ERR_ARG;
+  if (T == 0) return CW_OK;
+  dim3 grid(T), block(256);
+#define CW_LAUNCH(T_, WT_)                                                                                          \
+  hipLaunchKernelGGL((latent_store_kernel<T_, WT_>), grid, block, 0, stream, (const T_*)proj, stride, dq_off, nq, dkv_off, \
+                     rank, rot, rdims, (const WT_*)wq, (const WT_*)wkv, eps, positions, freq, slots, (T_*)cq, (T_*)plane,   \
+                     cache_rows)
+  if (dtype == CW_F32 && w_dtype == CW_F32) CW_LAUNCH(float, float);
+  else if (dtype == CW_BF16 && w_dtype == CW_BF16) CW_LAUNCH(bf16_t, bf16_t);
+  else if (dtype == CW_BF16 && w_dtype == CW_F32) CW_LAUNCH(bf16_t, float);
+  else return CW_ERR_DTYPE;
+#undef CW_LAUNCH
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- rotate one part of every head, to another layout
+// dst[t, h, dst_off + j] = src[t, h, src_off + j] for j < n, its first rdims elements rotated by
+// the token's position (pairs (i, i + rdims / 2), angle = float(position) * freq[i]). Tokens of src
+// and dst are src_stride / dst_stride elements apart, heads src_head / dst_head (token-major or
+// head-major alike; the host checks that the strides stay inside the tensors).
+template <typename T>
+__global__ void rotate_part_kernel(const T* __restrict__ src, int64_t src_stride, int64_t src_head, int src_off,
+                                   T* __restrict__ dst, int64_t dst_stride, int64_t dst_head, int dst_off, int heads, int n,
+                                   int rdims, const int* __restrict__ positions, const float* __restrict__ freq) {
+  const int64_t t = blockIdx.x;
+  const float pos = (float)positions[t];
+  const int half = rdims / 2;
+  for (int e = threadIdx.x; e < heads * n; e += blockDim.x) {
+    const int h = e / n, j = e % n;
+    const T* s = src + t * src_stride + h * src_head + src_off;
+    float v = cw_to_float(s[j]);
+    if (j < rdims) {
+      const int i = j < half ? j : j - half;
+      float sn, cs;
+      sincosf(pos * freq[i], &sn, &cs);
+      const float u = cw_to_float(s[i]), w = cw_to_float(s[i + half]);
+      v = j < half ? u * cs - w * sn : w * cs + u * sn;
+    }
+    dst[t * dst_stride + h * dst_head + dst_off + j] = cw_from_float<T>(v);
+  }
+}
+
+CW_EXPORT int cw_rotate_part(const void* src, int dtype, int64_t src_stride, int64_t src_head, int src_off, void* dst,
+                             int64_t dst_stride, int64_t dst_head, int dst_off, int heads, int n, int rdims,
+                             const int* positions, const float* freq, int T, hipStream_t stream) {
+  if (T < 0 || heads <= 0 || n < 0 || rdims < 0 || rdims > n || (rdims & 1)) return CW_ERR_ARG;
+  if (src_off < 0 || dst_off < 0 || src_stride < 1 || dst_stride < 1 || src_head < 1 || dst_head < 1) return CW_ERR_ARG;
+  if (!src || !dst || !positions || (rdims && !freq)) return CW_ERR_ARG;
+  if (T == 0 || n == 0) return CW_OK;
+  dim3 grid(T), block(256);
+  if (dtype == CW_F32)
+    hipLaunchKernelGGL(rotate_part_kernel<float>, grid, block, 0, stream, (const float*)src, src_stride, src_head, src_off,
+                       (float*)dst, dst_stride, dst_head, dst_off, heads, n, rdims, positions, freq);
+  else if (dtype == CW_BF16)
+    hipLaunchKernelGGL(rotate_part_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)src, src_stride, src_head, src_off,
+                       (bf16_t*)dst, dst_stride, dst_head, dst_off, heads, n, rdims, positions, freq);
+  else return CW_ERR_DTYPE;
   return cw_launch_status();
 }

@@ -126,6 +126,18 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_softcap": [P, L, F, P],
             "cw_rms_mean2": [P, P, P, P, I, F, P, I, I, I, P],
             "cw_qk_rownorm_store": [P, I, L, I, I, I, I, I, I, P, P, I, F, P, P, P, L, I, P],
+            "cw_add_dyt": [P, P, I, F, P, P, P, I, P, P, I, P, I, I, P],
+            "cw_gelu_erf": [P, I, L, P],
+            "cw_sigmoid_mul": [P, P, I, L, I, I, I, P],
+            "cw_bias_store": [P, I, L, I, I, I, I, I, I, P, I, P, P, P, L, I, P],
+            "cw_latent_store": [P, I, L, I, I, I, I, I, I, P, P, I, F, P, P, P, P, P, L, I, P],
+            "cw_rotate_part": [P, I, L, L, I, P, L, L, I, I, I, I, P, P, I, P],
+        },
+        "rows_attention": {
+            "cw_rows_attention_key_chunk": [I, I, I, I],
+            "cw_rows_attention_heads_per_group": [I, I, I],
+            "cw_rows_attention_tokens_per_item": [I, I, I],
+            "cw_rows_attention": [I, P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F, P],
         },
         "sink_attention": {
             "cw_sink_attention_max_bq": [I, I, I, I],
@@ -1542,3 +1554,200 @@ def sink_attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables
         _ptr(q), q_stride, _ptr(out), _ptr(k_cache), _ptr(v_cache), rows, _ptr(block_tables), block_tables.shape[1],
         _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(r1), _ptr(r2), _ptr(sink), _ptr(talk), heads, kv_heads, dim,
         vdim, block_size, int(window), float(scale), int(compute_units), _stream()), "sink_attention_prefill")
+
+
+# ---------------------------------------------------------------------------------------------
+class WithStreamInput:
+    """A pending branch output (or None) together with a float32 stream [T, H] that joins the
+    residual sum right after it: what a norm that ``accepts_stream_input`` adds before it norms.
+    The model hands it to the first norm of a run entry that begins a repeated pass."""
+
+    __slots__ = ("delta", "extra")
+
+    def __init__(self, delta, extra) -> None:
+        self.delta, self.extra = delta, extra
+
+
+def add_dynamic_tanh(resid, delta, delta_scale: float, extra, weight, bias, alpha, out, rows=None) -> torch.Tensor:
+    """resid += delta_scale * delta (+ extra), out = tanh(alpha * resid) * weight + bias, float32
+    inside; ``alpha`` is one float32 element on the device. With ``rows`` only those rows are
+    normed into out[i] and resid is left alone."""
+    _gpu(resid, delta, extra, weight, bias, alpha, out, rows)
+    T, H = resid.shape
+    _need(resid.dtype == torch.float32, "the residual stream is float32")
+    n = T if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, n, "rows")
+    _need(tuple(out.shape) == (n, H), f"out must be [{n}, {H}]")
+    _need(weight.numel() == H and (bias is None or (bias.numel() == H and bias.dtype == weight.dtype)),
+          "norm weight and bias must have the row's size and one type")
+    _need(alpha.dtype == torch.float32 and alpha.numel() == 1, "alpha must be one float32 element")
+    if delta is not None:
+        _need(tuple(delta.shape) == (T, H) and delta.dtype == out.dtype, "the pending branch must be [T, H] in the activation type")
+    if extra is not None:
+        _need(tuple(extra.shape) == (T, H) and extra.dtype == torch.float32, "the stream input must be [T, H] float32")
+    _check(_load("rowwise").cw_add_dyt(_ptr(resid), _ptr(delta), dtype_code(delta.dtype) if delta is not None else 0,
+                                       float(delta_scale), _ptr(extra), _ptr(weight), _ptr(bias), dtype_code(weight.dtype),
+                                       _ptr(alpha), _ptr(out), dtype_code(out.dtype), _ptr(rows), n, H, _stream()),
+           "add_dynamic_tanh")
+    return out
+
+
+def gelu_erf_(x: torch.Tensor) -> torch.Tensor:
+    """x <- 0.5 x (1 + erf(x / sqrt 2)), in place."""
+    _gpu(x)
+    _check(_load("rowwise").cw_gelu_erf(_ptr(x), dtype_code(x.dtype), x.numel(), _stream()), "gelu_erf")
+    return x
+
+
+def sigmoid_mul_(a: torch.Tensor, z: torch.Tensor, z_off: int) -> torch.Tensor:
+    """a[t, j] <- a[t, j] * sigmoid(z[t, z_off + j]), in place on ``a`` [T, n]; ``z`` [T, width]."""
+    _gpu(a, z)
+    T, n = a.shape
+    _need(z.dim() == 2 and z.shape[0] == T and z.dtype == a.dtype and 0 <= z_off and z_off + n <= z.shape[1],
+          "the gates must be [T, width] columns of the activations' type")
+    _check(_load("rowwise").cw_sigmoid_mul(_ptr(a), _ptr(z), dtype_code(a.dtype), z.shape[1], int(z_off), T, n, _stream()),
+           "sigmoid_mul")
+    return a
+
+
+def bias_store(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, nq: int, nk: int, nv: int, bias, slots,
+               k_plane, v_plane) -> None:
+    """Rows of ``proj`` [T, width] hold a token's query, key and value projections at the given
+    columns. ``bias`` ([width] or None) is added: queries in place, keys and values into the cache
+    rows ``k_plane[slots[t]]`` / ``v_plane[slots[t]]`` (flat [rows, nk] and [rows, nv]); a negative
+    slot writes nothing."""
+    _gpu(proj, bias, slots, k_plane, v_plane)
+    T, width = proj.shape
+    _i32(slots, T, "slots")
+    _need(bias is None or bias.numel() == width, "the bias must have one element per column of the projection")
+    _need(k_plane.dtype == proj.dtype and v_plane.dtype == proj.dtype, "cache and activations differ in type")
+    _need(k_plane.numel() % nk == 0 and v_plane.numel() % nv == 0 and k_plane.numel() // nk == v_plane.numel() // nv,
+          "key and value planes must hold the same number of rows")
+    _check(_load("rowwise").cw_bias_store(_ptr(proj), dtype_code(proj.dtype), width, q_off, k_off, v_off, nq, nk, nv,
+                                          _ptr(bias), dtype_code(bias.dtype) if bias is not None else 0, _ptr(slots),
+                                          _ptr(k_plane), _ptr(v_plane), k_plane.numel() // nk, T, _stream()), "bias_store")
+
+
+def latent_store(proj: torch.Tensor, dq_off: int, nq: int, dkv_off: int, rank: int, rot: int, rot_dims: int, q_weight,
+                 kv_weight, eps: float, positions, freq, slots, cq: torch.Tensor, plane) -> None:
+    """Rows of ``proj`` hold ``nq`` elements of a low-rank query step at ``dq_off`` and
+    ``rank + rot`` elements of the key/value one at ``dkv_off``: cq[t] = RMS(dq) * q_weight; the
+    cache row ``plane[slots[t]]`` ([rows, rank + rot]) gets RMS(dkv[:rank]) * kv_weight and then
+    the ``rot`` other elements, the first ``rot_dims`` of them rotated by the token's position
+    (half-split pairs, angle = position * freq[i], ``freq`` float32 [rot_dims / 2])."""
+    _gpu(proj, q_weight, kv_weight, positions, freq, slots, cq, plane)
+    T, width = proj.shape
+    _i32(positions, T, "positions")
+    _i32(slots, T, "slots")
+    _need(tuple(cq.shape) == (T, nq) and cq.dtype == proj.dtype, "cq must be [T, nq] in the activations' type")
+    _need(q_weight.numel() == nq and kv_weight.numel() == rank and q_weight.dtype == kv_weight.dtype, "norm weights must fit")
+    _need(plane.dtype == proj.dtype and plane.numel() % (rank + rot) == 0, "the plane must hold rows of rank + rot elements")
+    _need(rot_dims == 0 or (freq is not None and freq.dtype == torch.float32 and freq.numel() >= rot_dims // 2),
+          "freq must be float32 with rot_dims / 2 elements")
+    _check(_load("rowwise").cw_latent_store(_ptr(proj), dtype_code(proj.dtype), width, dq_off, nq, dkv_off, rank, rot, rot_dims,
+                                            _ptr(q_weight), _ptr(kv_weight), dtype_code(q_weight.dtype), float(eps),
+                                            _ptr(positions), _ptr(freq), _ptr(slots), _ptr(cq), _ptr(plane),
+                                            plane.numel() // (rank + rot), T, _stream()), "latent_store")
+
+
+def rotate_part(src: torch.Tensor, src_strides, src_off: int, dst: torch.Tensor, dst_strides, dst_off: int, heads: int,
+                n: int, rot_dims: int, positions, freq) -> None:
+    """dst(t, h, dst_off + j) = src(t, h, src_off + j) for j < n, the first ``rot_dims`` of them
+    rotated by the token's position (half-split pairs, angle = position * freq[i]). Element
+    (t, h, e) of a tensor lies at ``flatten()[t * strides[0] + h * strides[1] + e]``: token-major
+    and head-major tensors alike."""
+    _gpu(src, dst, positions, freq)
+    T = positions.numel()
+    _i32(positions, T, "positions")
+    _need(dst.dtype == src.dtype, "src and dst must be of one type")
+    for t, (st, sh), off in ((src, src_strides, src_off), (dst, dst_strides, dst_off)):
+        _need(st >= 1 and sh >= 1 and off >= 0 and (T == 0 or (T - 1) * st + (heads - 1) * sh + off + n <= t.numel()),
+              "rotate_part strides reach outside a tensor")
+    _need(rot_dims == 0 or (freq is not None and freq.dtype == torch.float32 and freq.numel() >= rot_dims // 2),
+          "freq must be float32 with rot_dims / 2 elements")
+    _check(_load("rowwise").cw_rotate_part(_ptr(src), dtype_code(src.dtype), int(src_strides[0]), int(src_strides[1]), src_off,
+                                           _ptr(dst), int(dst_strides[0]), int(dst_strides[1]), dst_off, heads, n, rot_dims,
+                                           _ptr(positions), _ptr(freq), T, _stream()), "rotate_part")
+
+
+MASK_KINDS = {"causal": 0, "window": 1, "segments": 2}
+
+
+def rows_attention_supported(heads: int, kv_heads: int, dim: int, vdim: int, maps: int = 1, alias: bool = False) -> bool:
+    lib = _load("rows_attention")
+    return bool(lib.cw_rows_attention_key_chunk(maps, dim, vdim, int(alias))
+                and lib.cw_rows_attention_heads_per_group(heads, kv_heads, maps))
+
+
+def rows_attention_tokens_per_item(heads: int, kv_heads: int, maps: int = 1) -> int:
+    """Tokens of one request that a work item of ``rows_attention`` may hold."""
+    return int(_load("rows_attention").cw_rows_attention_tokens_per_item(heads, kv_heads, maps))
+
+
+def heads_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[h] = x[h] @ weight[h].T for every head: ``x`` [heads, T, n_in], ``weight``
+    [heads, n_out, n_in], ``out`` [heads, T, n_out]; x and out may be views whose rows lie apart
+    (a slice of each head's columns), their last dimension dense. The library's batched product,
+    float32 accumulation (full float32 for float32 operands)."""
+    _need(x.dim() == 3 and weight.dim() == 3 and out.dim() == 3 and x.shape[0] == weight.shape[0] == out.shape[0]
+          and x.shape[2] == weight.shape[2] and out.shape[2] == weight.shape[1] and x.shape[1] == out.shape[1],
+          "heads_linear shapes")
+    _need(x.dtype == weight.dtype == out.dtype and x.stride(2) == 1 and out.stride(2) == 1, "heads_linear types and strides")
+    if x.shape[1]:
+        torch.bmm(x, weight.transpose(1, 2), out=out)
+    return out
+
+
+def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_tables, ctx_lens, cu_q, items, n_items: int,
+                   heads: int, kv_heads: int, dim: int, vdim: int, block_size: int, scale: float, maps: int = 1,
+                   mask: str = "causal", mask_size: int = 0, sink=None, lam=None, head_norm_eps=None,
+                   post_mult: float = 1.0) -> None:
+    """Softmax attention of the step's queries over paged rows. Query (t, head, map, d) lies at
+    ``q.flatten()[t * q_strides[0] + head * q_strides[1] + map * dim + d]``, output (t, head, c) at
+    ``out.flatten()[t * out_strides[0] + head * out_strides[1] + c]`` (token-major or head-major
+    tensors alike). ``k_plane`` [rows, >= kv_heads * maps * dim] holds a
+    token's keys [kv head][map][dim]; ``v_plane`` [rows, >= kv_heads * vdim] its values, or None:
+    the values are the first ``vdim`` elements of the key row (``maps`` 1).
+    ``mask``: "causal", "window" (the ``mask_size`` latest positions) or "segments" (the earlier
+    tokens of the token's segment of ``mask_size`` positions, segments counted from position 0).
+    ``sink`` float32 [heads]: exp(sink) joins the denominator. ``maps`` 2: the head's output is
+    map 0 minus ``lam`` (one float32 element) times map 1. ``head_norm_eps`` not None: the head's
+    output is divided by its root mean square and multiplied by ``post_mult``. ``items`` int32
+    [n_items, 4]: (request, first token, tokens, 0) with at most
+    ``rows_attention_tokens_per_item`` tokens each."""
+    alias = v_plane is None
+    _gpu(q, out, k_plane, v_plane, block_tables, ctx_lens, cu_q, items, sink, lam)
+    qs, qh = int(q_strides[0]), int(q_strides[1])
+    os_, oh = int(out_strides[0]), int(out_strides[1])
+    _need(out.dtype == q.dtype, "queries and output differ in type")
+    # the furthest element a token row of the step can touch must lie inside the tensors
+    def _fits(t, tok_stride, head_stride, width, tokens):
+        return tokens == 0 or (tokens - 1) * tok_stride + (heads - 1) * head_stride + width <= t.numel()
+    tokens = out.numel() // (heads * vdim)
+    _need(_fits(q, qs, qh, maps * dim, tokens) and _fits(out, os_, oh, vdim, tokens), "q / out strides reach outside the tensors")
+    k2 = k_plane.reshape(k_plane.shape[0], -1)
+    _need(k2.dtype == q.dtype and k2.shape[1] >= kv_heads * maps * dim, "the key plane must be [rows, >= kv_heads * maps * dim]")
+    rows = k2.shape[0]
+    v_row = 0
+    if not alias:
+        v2 = v_plane.reshape(v_plane.shape[0], -1)
+        _need(v2.dtype == q.dtype and v2.shape[0] == rows and v2.shape[1] >= kv_heads * vdim,
+              "the value plane must be [rows, >= kv_heads * vdim]")
+        v_row = v2.shape[1]
+    else:
+        _need(maps == 1 and kv_heads == 1 and vdim <= dim, "values inside the key row: one map, one key/value head, vdim <= dim")
+    R = ctx_lens.numel()
+    _i32(ctx_lens, R, "ctx_lens")
+    _i32(cu_q, R + 1, "cu_q")
+    _i32(items, 4 * n_items, "items")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= R, "block tables must be int32 [R, width]")
+    _need(sink is None or (sink.dtype == torch.float32 and sink.numel() == heads), f"sink must be float32 with {heads} elements")
+    _need((maps == 1 and lam is None) or (maps == 2 and lam is not None and lam.dtype == torch.float32 and lam.numel() == 1),
+          "two maps take one float32 lambda, one map none")
+    _need(mask in MASK_KINDS and (mask == "causal" or mask_size >= 1), f"mask {mask!r} of size {mask_size}")
+    _check(_load("rows_attention").cw_rows_attention(
+        dtype_code(q.dtype), _ptr(q), qs, qh, _ptr(out), os_, oh, _ptr(k_plane), _ptr(k_plane if alias else v_plane), k2.shape[1],
+        v_row, rows, _ptr(block_tables), block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(sink),
+        _ptr(lam), heads, kv_heads, dim, vdim, maps, block_size, MASK_KINDS[mask], int(mask_size), float(scale),
+        0 if head_norm_eps is None else 1, float(head_norm_eps or 0.0), float(post_mult), _stream()), "rows_attention")

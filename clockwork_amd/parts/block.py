@@ -10,22 +10,26 @@ class PreNormBlock:
 
     The residual stream is float32 and is only ever touched by the norms' fused add, so
     each branch output is added exactly once, in float32. ``forward`` takes the previous
-    block's pending output ``delta`` and returns its own.
+    block's pending output ``delta`` and returns its own. A block without a feed-forward (and
+    without its norm) is the first half alone.
     """
 
-    def __init__(self, mixer, feed_forward, mixer_norm, ffn_norm) -> None:
+    def __init__(self, mixer, mixer_norm, feed_forward=None, ffn_norm=None) -> None:
+        if (feed_forward is None) != (ffn_norm is None):
+            raise ValueError("a pre-norm block has a feed-forward and its norm, or neither")
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.mixer_norm = mixer_norm
         self.ffn_norm = ffn_norm
 
     def parts(self) -> dict:
-        return {
-            "mixer": self.mixer,
-            "feed_forward": self.feed_forward,
-            "mixer_norm": self.mixer_norm,
-            "ffn_norm": self.ffn_norm,
-        }
+        parts = {"mixer": self.mixer}
+        if self.feed_forward is not None:
+            parts["feed_forward"] = self.feed_forward
+        parts["mixer_norm"] = self.mixer_norm
+        if self.ffn_norm is not None:
+            parts["ffn_norm"] = self.ffn_norm
+        return parts
 
     def first_norm(self):
         """The norm that takes what the block before hands on (may it be two pending outputs?)."""
@@ -34,6 +38,8 @@ class PreNormBlock:
     def forward(self, resid, delta, ctx, cache):
         x = self.mixer_norm.forward(resid, delta)
         a = self.mixer.forward(x, ctx, cache)
+        if self.feed_forward is None:
+            return a
         # Few rows: the second norm can run inside the feed-forward's first product, which saves a
         # launch. That kernel writes no residual, so the mixer's output stays pending and is
         # handed on together with the feed-forward's (the next norm must be able to take both).

@@ -1,0 +1,93 @@
+"""Attention with two score maps a head over shared values (``DifferentialAttentionSpec``).
+
+Steps: one fused q/k/v product; one kernel adds the biases, rewrites the queries and writes keys
+and values to their pages (every token of the step is cached before any query reads); the
+attention kernel runs both maps of a head in one workgroup, subtracts the second from the first
+with the layer's lambda, norms the head's output and scales it; output product. Keys
+[kv_heads, 2, key_dim] and values [kv_heads, value_dim] are two planes of a ``PagedRowsSpec``;
+with a segment mask the pages before the running segment are given back while the request runs.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from clockwork_amd import ops
+from clockwork_amd.config.spec import PagedRowsSpec, ParamSpec
+from clockwork_amd.parts.base import EntryCache, Part
+from clockwork_amd.parts.sink_attention import query_runs
+from clockwork_amd.parts.specs import DifferentialAttentionSpec
+
+MAPS = 2
+
+
+class DifferentialAttention(Part):
+    graph_safe = True
+
+    def __init__(self, spec: DifferentialAttentionSpec) -> None:
+        self.spec = spec
+        self.q_width = spec.num_heads * MAPS * spec.key_dim
+        self.k_width = spec.num_kv_heads * MAPS * spec.key_dim
+        self.v_width = spec.num_kv_heads * spec.value_dim
+
+    def param_specs(self):
+        s = self.spec
+        width = self.q_width + self.k_width + self.v_width
+        specs = {
+            "qkv_weight": ParamSpec((width, s.hidden_size)),
+            "out_weight": ParamSpec((s.hidden_size, s.num_heads * s.value_dim)),
+        }
+        if s.qkv_bias:
+            specs["qkv_bias"] = ParamSpec((width,), precision="stored", init=("normal", 0.02))
+        for name in ("lq1", "lk1", "lq2", "lk2"):
+            specs[name] = ParamSpec((s.key_dim,), precision="float32", init=("normal", 0.1))
+        return specs
+
+    def cache_need(self):
+        s = self.spec
+        return PagedRowsSpec((("k", (s.num_kv_heads, MAPS * s.key_dim)), ("v", (s.num_kv_heads, s.value_dim))),
+                             window=s.window, segment=s.segment)
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None), ("rows_attention", None)]
+
+    def mask(self) -> tuple:
+        s = self.spec
+        if s.segment is not None:
+            return "segments", s.segment
+        return ("window", s.window) if s.window is not None else ("causal", 0)
+
+    def bind(self, params, device, dtype) -> None:
+        s = self.spec
+        self.qkv_weight, self.qkv_bias = params["qkv_weight"], params.get("qkv_bias")
+        self.out_weight = params["out_weight"]
+        # lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + lambda_init: one float32 number a layer
+        lam = (torch.exp((params["lq1"].float() * params["lk1"].float()).sum())
+               - torch.exp((params["lq2"].float() * params["lk2"].float()).sum()) + s.lambda_init)
+        self.lam = lam.reshape(1).to(device=device, dtype=torch.float32).contiguous()
+        self.dtype = dtype
+        if not ops.rows_attention_supported(s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim, maps=MAPS):
+            raise ValueError(f"two-map attention with keys of {s.key_dim} and values of {s.value_dim} elements is beyond "
+                             "the attention kernel for paged rows (value_dim up to 512, tiles of 150 KB of LDS)")
+        self.run = ops.rows_attention_tokens_per_item(s.num_heads, s.num_kv_heads, MAPS)
+
+    def prepare(self, ctx) -> None:
+        query_runs(ctx, self.run)
+
+    def forward(self, x: torch.Tensor, ctx, cache: EntryCache) -> torch.Tensor:
+        s = self.spec
+        policy = getattr(ctx, "products", None)
+        if not cache.writes:
+            raise NotImplementedError("this mixer writes its own keys and values: it cannot borrow another entry's cache")
+        k_plane, v_plane = cache.planes["k"], cache.planes["v"]
+        qkv = ops.linear(x, self.qkv_weight, policy=policy)
+        ops.bias_store(qkv, 0, self.q_width, self.q_width + self.k_width, self.q_width, self.k_width, self.v_width,
+                       self.qkv_bias, ctx.slots[cache.group], k_plane, v_plane)
+        out = torch.empty((x.shape[0], s.num_heads * s.value_dim), dtype=x.dtype, device=x.device)
+        items, n_items = query_runs(ctx, self.run)
+        kind, size = self.mask()
+        ops.rows_attention(qkv, (qkv.shape[1], MAPS * s.key_dim), out, (out.shape[1], s.value_dim), k_plane, v_plane,
+                           ctx.block_tables[cache.group], ctx.ctx_lens, ctx.cu_q, items, n_items, s.num_heads, s.num_kv_heads,
+                           s.key_dim, s.value_dim, cache.block_size, s.scale, maps=MAPS, mask=kind, mask_size=size, lam=self.lam,
+                           head_norm_eps=s.norm_eps, post_mult=1.0 - s.lambda_init)
+        return ops.linear(out, self.out_weight, policy=policy)

@@ -65,3 +65,28 @@ class GatedMLP(Part):
         gate_up = ops.linear(x, self.gate_up, policy=policy)
         inner = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
         return ops.linear(ops.gelu_tanh_mul(gate_up, inner), self.down, policy=policy)
+
+
+class DenseMLP(Part):
+    """down(gelu(up(x))) (``DenseMLPSpec``): the up product, the erf GELU in place (float32
+    inside), the down product."""
+
+    graph_safe = True
+
+    def __init__(self, spec) -> None:
+        self.spec = spec
+
+    def param_specs(self):
+        H, I = self.spec.hidden_size, self.spec.intermediate_size
+        return {"up_weight": ParamSpec((I, H)), "down_weight": ParamSpec((H, I))}
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None)]
+
+    def bind(self, params, device, dtype) -> None:
+        self.up = params["up_weight"]
+        self.down = params["down_weight"]
+
+    def forward(self, x, ctx) -> torch.Tensor:
+        policy = getattr(ctx, "products", None)
+        return ops.linear(ops.gelu_erf_(ops.linear(x, self.up, policy=policy)), self.down, policy=policy)

@@ -12,6 +12,7 @@ from typing import Optional
 
 import torch
 
+from clockwork_amd import ops
 from clockwork_amd.config.spec import ModelSpec, ParamSpec
 from clockwork_amd.parts.specs import LinearHeadSpec, TokenEmbeddingSpec
 from clockwork_amd.registry import build_arrangement, build_part
@@ -57,6 +58,12 @@ class DecoderModel:
         self.layers = _build_layers(spec)
         self.final_norm = build_part(spec.final_norm)
         self.head = build_part(_head_spec(spec))
+        for i, entry in enumerate(spec.run):
+            if entry.add_input:
+                first_norm = getattr(self.layers[entry.layer], "first_norm", None)
+                if not getattr(first_norm() if first_norm is not None else None, "accepts_stream_input", False):
+                    raise ValueError(f"run[{i}] adds the model's input to the stream again, which the first norm of "
+                                     f"layer {entry.layer} cannot take (no accepts_stream_input)")
 
     def named_parts(self) -> list:
         return _named_parts(self.embedding, self.layers, self.final_norm, self.head)
@@ -145,9 +152,15 @@ class DecoderModel:
         if positions_of is not None:
             ctx.positions = positions_of(ctx)
         resid = self.embedding.forward(ctx)
+        # a run entry that is fed the model's input again needs it as it was: the stream is updated
+        # in place, so the embedding part makes it a second time (a gather, and a kernel launch
+        # like any other for a step that is captured as a graph)
+        again = self.embedding.forward(ctx) if any(e.add_input for e in self.spec.run) else None
         delta = None
         run = self.spec.run
         for i, entry in enumerate(run):
+            if entry.add_input:
+                delta = ops.WithStreamInput(delta, again)
             # may this block hand on two pending outputs? Only if the norm that takes them next (the
             # next block's first norm, as that block's arrangement names it, or the final norm) can
             if i + 1 < len(run):

@@ -68,3 +68,43 @@ class LayerNorm(Part):
         n = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.spec.size), dtype=self.dtype, device=resid.device)
         return ops.add_layernorm(resid, delta, self.weight, self.bias, self.spec.eps, out, rows)
+
+
+class DynamicTanh(Part):
+    """tanh(alpha * x) * weight + bias (``DynamicTanhSpec``), fused with the residual add: the
+    pending branch output joins the float32 stream multiplied by the spec's ``delta_scale``, and
+    after it a second float32 stream when the model hands one on (``ops.WithStreamInput``)."""
+
+    graph_safe = True
+    accepts_stream_input = True
+
+    def __init__(self, spec) -> None:
+        self.spec = spec
+
+    def param_specs(self):
+        specs = {"weight": ParamSpec((self.spec.size,), precision="stored", init=("one_plus_uniform", 0.1)),
+                 "alpha": ParamSpec((1,), precision="float32", init=("uniform", 0.3, 1.0))}
+        if self.spec.bias:
+            specs["bias"] = ParamSpec((self.spec.size,), precision="stored", init=("normal", 0.02))
+        return specs
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None)]
+
+    def bind(self, params, device, dtype) -> None:
+        self.weight = params["weight"]
+        self.bias = params.get("bias")
+        if self.bias is not None and self.bias.dtype != self.weight.dtype:
+            self.bias = self.bias.to(self.weight.dtype)
+        self.alpha = params["alpha"].reshape(1)
+        self.dtype = dtype
+
+    def forward(self, resid: torch.Tensor, delta, rows=None) -> torch.Tensor:
+        extra = None
+        if isinstance(delta, ops.WithStreamInput):
+            delta, extra = delta.delta, delta.extra
+        if isinstance(delta, ops.PartialSums):
+            delta = delta.sum(self.dtype)
+        n = resid.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.spec.size), dtype=self.dtype, device=resid.device)
+        return ops.add_dynamic_tanh(resid, delta, self.spec.delta_scale, extra, self.weight, self.bias, self.alpha, out, rows)

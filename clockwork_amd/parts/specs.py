@@ -201,3 +201,99 @@ class BranchGateSpec:
 
     hidden_size: int
     branches: int = 2
+
+
+@dataclass(frozen=True)
+class DynamicTanhSpec:
+    """y = tanh(alpha * x) * weight + bias with one learned scalar alpha: a norm that takes no mean
+    or variance of the row. ``delta_scale``: what the norm adds to the residual stream first (the
+    pending branch output) is multiplied by it (a model-wide residual multiplier)."""
+
+    size: int
+    delta_scale: float = 1.0
+    bias: bool = True
+
+
+@dataclass(frozen=True)
+class DenseMLPSpec:
+    """down(act(up(x))), no gate, no biases; ``activation`` "gelu" (the erf form)."""
+
+    hidden_size: int
+    intermediate_size: int
+    activation: str = "gelu"
+
+    def __post_init__(self):
+        if self.activation not in ("gelu",):
+            raise ValueError(f"activation {self.activation!r}: expected 'gelu'")
+
+
+@dataclass(frozen=True)
+class DifferentialAttentionSpec:
+    """Grouped softmax attention in which every query head has two score maps over the same
+    values: queries [heads, 2, key_dim], keys [kv_heads, 2, key_dim], values [kv_heads, value_dim],
+    all from biased projections (``qkv_bias``). The head's output is A_1 - lambda * A_2 with
+    lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + ``lambda_init`` (four learned vectors of key_dim, one
+    number a layer), then divided by its root mean square over value_dim (``norm_eps`` inside the
+    root, no weight) and multiplied by 1 - ``lambda_init``. No position encoding.
+
+    What a token sees: ``segment`` S: the earlier tokens of its own run of S positions (runs
+    counted from position 0); ``window`` W: itself and the W - 1 before it; neither: all earlier ones."""
+
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    scale: float
+    lambda_init: float
+    norm_eps: float
+    segment: Optional[int] = None
+    window: Optional[int] = None
+    qkv_bias: bool = True
+
+    def __post_init__(self):
+        if self.num_heads < 1 or self.num_kv_heads < 1 or self.num_heads % self.num_kv_heads:
+            raise ValueError(f"num_heads {self.num_heads} is not a multiple of num_kv_heads {self.num_kv_heads}")
+        if self.key_dim < 1 or self.value_dim < 1:
+            raise ValueError("key_dim and value_dim must be positive")
+        if self.segment is not None and self.window is not None:
+            raise ValueError("an attention mask has segments or a window, not both")
+        for name in ("segment", "window"):
+            if getattr(self, name) is not None and getattr(self, name) < 1:
+                raise ValueError(f"{name} must be positive, got {getattr(self, name)}")
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose keys and values are made from one cached latent a token. Queries:
+    RMS-normed low-rank step of ``q_rank``, then [heads, key_dim + rope_dim]. Keys/values: a
+    projection to ``kv_rank + rope_dim`` elements; the first kv_rank, RMS-normed with a weight, are
+    the latent c, the others one rotated key part that all heads share. Head a's key is
+    [uk_a c, rotated part], its value uv_a c (value_dim). The rope_dim parts of queries and keys
+    are rotated by position: the first ``rotary_dims`` of them in half-split pairs with base
+    ``rope_base``. ``sink``: exp(sink[a]) joins head a's softmax denominator. ``output_gate``: the
+    concatenated heads are multiplied by the sigmoid of a projection of the mixer's input.
+    Only the latent and the rotated part are cached: kv_rank + rope_dim elements a token."""
+
+    hidden_size: int
+    num_heads: int
+    key_dim: int
+    rope_dim: int
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    rope_base: float
+    rotary_dims: int
+    norm_eps: float
+    sink: bool = True
+    output_gate: bool = True
+    window: Optional[int] = None
+
+    def __post_init__(self):
+        if min(self.num_heads, self.key_dim, self.value_dim, self.q_rank, self.kv_rank) < 1 or self.rope_dim < 0:
+            raise ValueError("heads, key_dim, value_dim, q_rank and kv_rank must be positive, rope_dim not negative")
+        if self.rotary_dims % 2 or not 0 <= self.rotary_dims <= self.rope_dim:
+            raise ValueError(f"rotary_dims {self.rotary_dims} must be even and at most rope_dim {self.rope_dim}")
+        if self.window is not None and self.window < 1:
+            raise ValueError(f"window must be positive, got {self.window}")

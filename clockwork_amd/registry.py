@@ -39,6 +39,7 @@ _BUILTIN_ARCHITECTURES = {
     "Qwen2ForCausalLM": "clockwork_amd.models.qwen2",
     "qwen2": "clockwork_amd.models.qwen2",
     "Fuvavik": "clockwork_amd.models.fuvavik",
+    "Pesorax": "clockwork_amd.models.pesorax",
 }
 
 
@@ -98,6 +99,10 @@ _BUILTIN_PARTS = {
     "DecayedLinearAttentionSpec": ("clockwork_amd.parts.linear_attention", "DecayedLinearAttention"),
     "PairMixerSpec": ("clockwork_amd.parts.pair", "PairMixer"),
     "BranchGateSpec": ("clockwork_amd.parts.block", "BranchGate"),
+    "DynamicTanhSpec": ("clockwork_amd.parts.norm", "DynamicTanh"),
+    "DenseMLPSpec": ("clockwork_amd.parts.mlp", "DenseMLP"),
+    "DifferentialAttentionSpec": ("clockwork_amd.parts.differential_attention", "DifferentialAttention"),
+    "LatentAttentionSpec": ("clockwork_amd.parts.latent_attention", "LatentAttention"),
 }
 _ARRANGEMENTS: dict[str, Callable[..., Any]] = {}
 _BUILTIN_ARRANGEMENTS = {"prenorm": ("clockwork_amd.parts.block", "PreNormBlock"),

@@ -32,7 +32,13 @@ def _split_rows(t, index: int, parts: int):
     return t[index * rows : (index + 1) * rows]
 
 
+def _as_vector(t):
+    """A scalar (or anything else) as a 1-d tensor: a parameter that the file holds with shape ()."""
+    return t.reshape(-1)
+
+
 register_transform("transpose", _transpose)
+register_transform("as_vector", _as_vector)
 register_transform("split_rows", _split_rows)
 
 
