@@ -71,7 +71,7 @@ __global__ __launch_bounds__(256) void rows_attention_kernel(const RowsAttnParam
 
   const int tid = threadIdx.x, row = tid >> 4, sub = tid & 15;
   const int* item = p.items + 4 * (int64_t)blockIdx.x;
-  const int req = item[0], tok0 = item[1], ntok = item[2];
+  const int req = item[0], tok0 = item[1];
   const int g = blockIdx.y;                             // key/value head
   const int group = p.heads / p.kv_heads;
   const int HC = p.heads_per_group;
@@ -80,6 +80,8 @@ __global__ __launch_bounds__(256) void rows_attention_kernel(const RowsAttnParam
   const int rows_per_token = HC * M;
   const int ctx = p.ctx_lens[req];
   const int q_len = p.cu_q[req + 1] - p.cu_q[req];
+  if (tok0 >= q_len) return;  // an item past the request's tokens (a batch of fixed shape)
+  const int ntok = min(min(item[2], p.tokens_per_item), q_len - tok0);
   const int pos0 = ctx - q_len + tok0;                  // position of the item's first token
   // this thread's row
   const int tl = row / rows_per_token, hl = (row % rows_per_token) / M, m = row % M;
@@ -196,7 +198,7 @@ __global__ __launch_bounds__(256) void rows_attention_kernel(const RowsAttnParam
     }
   }
   // a row that saw no key and has no sink cannot happen: every token sees itself
-  const float inv = 1.0f / run_sum;
+  const float inv = run_sum > 0.0f ? 1.0f / run_sum : 0.0f;
   const float lam = (M == 2 && p.lambda) ? p.lambda[0] : 0.0f;
   float sq = 0.0f;
 #pragma unroll

@@ -136,3 +136,68 @@ FUVAVIK_LONG = {
 }
 # name -> (config, weight seed, cache block size)
 FUVAVIK_CONFIGS = {"FA": (FUVAVIK_A, 21, 8), "FB": (FUVAVIK_B, 22, 16), "FC": (FUVAVIK_C, 23, 4)}
+
+
+# ---- Pesorax: small models that differ in every size and constant; layers of one model differ too.
+def _pesorax_attention(heads, kv_heads, dim, vdim, scale, diff, segment, ff):
+    return {"type": "attention",
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "diff": diff,
+                      "mask": {"size": segment}},
+            "mlp": None if ff is None else {"kind": "dense", "ff": ff}}
+
+
+def _pesorax_latent(heads, dim, rot_dim, rot_dims, vdim, q_rank, kv_rank, scale, base, ff):
+    return {"type": "latent_attention",
+            "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
+                      "scale": scale, "rot": {"base": base, "dims": rot_dims}},
+            "mlp": None if ff is None else {"kind": "dense", "ff": ff}}
+
+
+# four layers that share nothing; the middle two run twice; three query heads a key/value head,
+# segments of 9 and 33, a rope part of which only half is rotated, a layer without a feed-forward
+PESORAX_A = {
+    "architecture": "Pesorax", "vocab": 300, "width": 96, "residual_mult": 0.5, "norm": {"eps": 1e-5},
+    "loop": {"start": 1, "stop": 3, "times": 2},
+    "layers": [
+        _pesorax_attention(6, 2, 16, 24, 0.2, 0.3, 9, 72),
+        _pesorax_latent(3, 24, 16, 8, 20, 40, 48, 0.15, 100.0, None),
+        _pesorax_attention(2, 2, 8, 8, 0.3, 0.8, 33, 40),
+        _pesorax_latent(2, 16, 8, 8, 32, 24, 16, 0.2, 10000.0, 64),
+    ],
+}
+# a width that is no multiple of 8, no repeated layers (no "loop" key at all), one key/value head
+# for three query heads, a segment longer than any request of the tests (every earlier key is
+# seen) and one of 1 (a token sees itself alone), a residual multiplier of 1
+PESORAX_B = {
+    "architecture": "Pesorax", "vocab": 127, "width": 100, "residual_mult": 1.0, "norm": {"eps": 3e-4},
+    "layers": [
+        _pesorax_attention(3, 1, 40, 24, 0.16, 0.5, 300, 50),
+        _pesorax_latent(5, 8, 4, 4, 12, 20, 36, 0.3, 50.0, 130),
+        _pesorax_attention(2, 1, 8, 32, 0.35, 0.1, 1, None),
+    ],
+}
+# one head everywhere, sizes of 1 and 2 where the design allows them, the whole model repeated
+# three times
+PESORAX_C = {
+    "architecture": "Pesorax", "vocab": 64, "width": 48, "residual_mult": 0.25, "norm": {"eps": 1e-6},
+    "loop": {"start": 0, "stop": 2, "times": 3},
+    "layers": [
+        _pesorax_latent(1, 2, 2, 2, 1, 4, 8, 0.5, 4.0, 24),
+        _pesorax_attention(1, 1, 32, 8, 0.18, 0.6, 17, 24),
+    ],
+}
+# layers of unlike sizes for long requests: segments of 77 to 1500, a latent of 256 + 64 elements,
+# sizes that the matrix cores take and sizes that they do not
+PESORAX_LONG = {
+    "architecture": "Pesorax", "vocab": 211, "width": 192, "residual_mult": 0.4, "norm": {"eps": 2e-6},
+    "loop": {"start": 0, "stop": 1, "times": 2},
+    "layers": [
+        _pesorax_attention(6, 3, 32, 48, 0.3, 0.4, 200, 384),
+        _pesorax_latent(8, 64, 32, 32, 64, 96, 256, 0.2, 10000.0, None),
+        _pesorax_attention(8, 2, 64, 128, 0.15, 0.7, 1500, 100),
+        _pesorax_latent(16, 32, 64, 32, 32, 64, 128, 0.25, 500.0, 64),
+        _pesorax_attention(4, 4, 64, 64, 0.2, 0.2, 77, None),
+    ],
+}
+# name -> (config, weight seed, cache block size)
+PESORAX_CONFIGS = {"PA": (PESORAX_A, 31, 8), "PB": (PESORAX_B, 32, 16), "PC": (PESORAX_C, 33, 4)}
