@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16] [--shape 1.5b]
     python bench.py --workload mixed|arrivals|agent [--shape 7b] [--requests 64]
-    python bench.py --design fuvavik [--size s|m|l] [--layers L] [--batch B]
+    python bench.py --design fuvavik|pesorax [--size s|m|l] [--layers L] [--batch B]
 
 Default workload: the layer sizes of Qwen2.5-1.5B with random weights (seed 2), bfloat16,
 8 requests that each hold a 2048-token prompt, context limit 4096, pages of 16 tokens. A
@@ -520,11 +520,51 @@ def fuvavik_config(size: dict, layers: int, max_positions: int) -> dict:
             "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "layers": [layer] * layers}
 
 
+# Layer sizes for ``--design pesorax``: the same widths, head counts and feed-forwards; the two-map
+# attention with key rows of 64 elements a map and values of the Qwen2 head's size (``head_dim``:
+# what the Qwen2 model beside it gets) and segments of half the prompt, the latent attention with a latent of 512 + 64 elements a token,
+# low-rank queries and per-head keys of 128 + 64 and values of 128. Layers alternate between the
+# two kinds; the first two run twice (``layers`` counts layer runs: the Qwen2 model beside it has
+# that many layers).
+PESORAX_SIZES = {
+    "s": dict(width=896, heads=14, kv_heads=2, dim=64, vdim=64, head_dim=64, segment=1024, l_heads=14, l_dim=64, l_rot=64,
+              l_vdim=64, q_rank=384, kv_rank=256, ff=4864, layers=6),
+    "m": dict(width=1536, heads=12, kv_heads=2, dim=64, vdim=128, head_dim=128, segment=1024, l_heads=12, l_dim=128, l_rot=64,
+              l_vdim=128, q_rank=768, kv_rank=512, ff=8960, layers=6),
+    "l": dict(width=2048, heads=16, kv_heads=2, dim=64, vdim=128, head_dim=128, segment=1024, l_heads=16, l_dim=128, l_rot=64,
+              l_vdim=128, q_rank=1024, kv_rank=512, ff=11008, layers=6),
+}
+
+
+def pesorax_config(size: dict, layers: int, max_positions: int) -> dict:
+    attention = {
+        "type": "attention",
+        "mixer": {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"],
+                  "scale": size["dim"] ** -0.5, "diff": 0.5, "mask": {"size": size["segment"]}},
+        "mlp": {"kind": "dense", "ff": size["ff"]},
+    }
+    latent = {
+        "type": "latent_attention",
+        "mixer": {"heads": size["l_heads"], "dim": size["l_dim"], "rot_dim": size["l_rot"], "vdim": size["l_vdim"],
+                  "q_rank": size["q_rank"], "kv_rank": size["kv_rank"], "scale": (size["l_dim"] + size["l_rot"]) ** -0.5,
+                  "rot": {"base": 10000.0, "dims": size["l_rot"]}},
+        "mlp": {"kind": "dense", "ff": size["ff"]},
+    }
+    # ``layers`` layer runs: the first two layers twice, the others once
+    distinct = max(2, layers - 2)
+    return {"architecture": "Pesorax", "vocab": DESIGN_VOCAB, "width": size["width"], "residual_mult": 0.5,
+            "norm": {"eps": 1e-6}, "loop": {"start": 0, "stop": 2, "times": 2 if layers >= 4 else 1},
+            "layers": [attention if i % 2 == 0 else latent for i in range(distinct)]}
+
+
+DESIGNS = {"fuvavik": (FUVAVIK_SIZES, fuvavik_config), "pesorax": (PESORAX_SIZES, pesorax_config)}
+
+
 def qwen2_config_like(size: dict, layers: int, max_positions: int) -> dict:
     """The closest model the engine had before: Qwen2 blocks of the same width, heads, head size,
     feed-forward, layers and vocabulary."""
     return dict(QWEN25_1P5B, vocab_size=DESIGN_VOCAB, hidden_size=size["width"], num_hidden_layers=layers,
-                num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
+                num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size.get("head_dim", size["dim"]),
                 intermediate_size=size["ff"], max_position_embeddings=max_positions, tie_word_embeddings=True)
 
 
@@ -537,13 +577,14 @@ def run_design(args) -> dict:
     from clockwork_amd.config.engine import EngineConfig
     from clockwork_amd.engine.model_runner import GRAPH_BATCH_SIZES, ModelRunner
 
-    size = FUVAVIK_SIZES[args.size]
+    sizes, make_config = DESIGNS[args.design]
+    size = sizes[args.size]
     layers = args.layers if args.layers is not None else size["layers"]
     context = context_of(args)
     out = {"design": args.design, "size": {**size, "layers": layers, "vocab": DESIGN_VOCAB}, "dtype": args.dtype,
            "prompt_len": args.prompt_len, "batch": args.batch, "steps": args.steps,
            "data": "synthetic: uniform random token ids, random weights (seed 2)"}
-    configs = {args.design: fuvavik_config(size, layers, context), "qwen2 of equal size": qwen2_config_like(size, layers, context)}
+    configs = {args.design: make_config(size, layers, context), "qwen2 of equal size": qwen2_config_like(size, layers, context)}
     for name, config in configs.items():
         cfg = EngineConfig.defaults(
             f"random:{name}", dtype=args.dtype, max_model_len=context, block_size=BLOCK,
@@ -607,7 +648,7 @@ def main() -> int:
     ap.add_argument("--peaks", action="store_true", help="measure a device copy and a large library product instead")
     ap.add_argument("--decode-attention-grid", action="store_true",
                     help="time the attention part alone over the reference's grid of batch sizes and context lengths instead")
-    ap.add_argument("--design", default=None, choices=("fuvavik",),
+    ap.add_argument("--design", default=None, choices=sorted(DESIGNS),
                     help="measure another design's prefill and decode beside the Qwen2 model of equal size instead")
     ap.add_argument("--size", default="m", choices=sorted(FUVAVIK_SIZES), help="--design: which layer sizes")
     ap.add_argument("--temperature", type=float, default=0.0, help="sample instead of the greedy decoding of the recorded benchmark")

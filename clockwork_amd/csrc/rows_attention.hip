@@ -296,3 +296,475 @@ CW_EXPORT int cw_rows_attention(int dtype, const void* q, int64_t q_stride, int6
 #undef CW_LAUNCH
   return cw_launch_status();
 }
+
+// ======================================================================================
+// bfloat16 on the matrix cores, for portions and single tokens alike.
+//
+// A workgroup takes up to 16 tokens of one request (the 16 columns of its score tiles), one
+// key/value head, up to four (two maps) or 4 * UPW (one map) query heads of that head's group,
+// VW = 16 * NT of the value columns, and one of gridDim.z runs of the keys. A wave holds UPW
+// "units": with two maps the two maps of one head, else UPW heads. Keys come in chunks of 32
+// through LDS (row-major for the scores, the values transposed for the value product); the next
+// chunk is fetched into registers while this one is multiplied.
+//
+// Scores are made as K Q^T (v_mfma_f32_16x16x32_bf16): a lane then holds, for ITS query
+// (lane % 16), the keys 4 * slot + e and 16 + 4 * slot + e of the chunk (slot = lane / 16), which is
+// the A operand of the value product as it lies in the registers; the value fragments are read
+// with the keys in that order. Softmax in units of log 2 with a running maximum per query, float32;
+// the weights enter the value product rounded to bfloat16, sums are float32.
+//
+// With one run of keys the workgroup finishes its heads itself (denominator, the two maps'
+// difference, the head norm); with several, every run leaves maximum, denominator and
+// unnormalised sums in a workspace and rows_merge_kernel finishes.
+// ======================================================================================
+typedef __attribute__((ext_vector_type(8))) __bf16 ra_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float ra_f32x4_t;
+#define RM_KT 32
+
+__device__ __forceinline__ ra_bf16x8_t ra_load8(const bf16_t* p) { return *reinterpret_cast<const ra_bf16x8_t*>(p); }
+
+struct RowsMfmaExtra {
+  float* workspace;     // [items][gridDim.y][runs][4 waves][UPW][16 queries][2 + VW] when runs > 1
+  int head_chunks;      // workgroups that share the heads of a key/value head's group
+  int v_splits;         // workgroups that share the value columns
+  int heads_per_wg;     // 4 (two maps) or 4 * UPW
+};
+
+__device__ __forceinline__ int ra_oldest_seen(int kind, int size, int pos) {
+  if (kind == RA_MASK_WINDOW) return max(0, pos - size + 1);
+  if (kind == RA_MASK_SEGMENTS) return (pos / size) * size;
+  return 0;
+}
+
+template <int D32, int NT, int UPW, int MAPS>
+__global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, const RowsMfmaExtra x) {
+  extern __shared__ __align__(16) unsigned char ra_smem[];
+  constexpr int D = D32 * 32, DA = D * MAPS, VW = NT * 16;
+  constexpr int KROW = DA + 8, VROW = RM_KT + 8;
+  constexpr int KPR = DA / 8, VPR = VW / 8;
+  constexpr int PFK = (RM_KT * KPR + 255) / 256, PFV = (RM_KT * VPR + 255) / 256;
+  static_assert(MAPS == 1 || UPW == 2, "two maps: a wave holds the two maps of one head");
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l16 = lane & 15, slot = lane >> 4;
+  const int* item = p.items + 4 * (int64_t)blockIdx.x;
+  const int req = item[0], tok0 = item[1];
+  const int q_len = p.cu_q[req + 1] - p.cu_q[req];
+  if (tok0 >= q_len) return;  // an item past the request's tokens (a batch of fixed shape)
+  const int nq = min(min(item[2], 16), q_len - tok0);
+  const int pos0 = p.ctx_lens[req] - q_len + tok0;
+  const int last = pos0 + nq - 1;
+  const int first = ra_oldest_seen(p.mask_kind, p.mask_size, pos0);
+  const int lo_last = ra_oldest_seen(p.mask_kind, p.mask_size, last);
+  const int64_t row0 = (int64_t)p.cu_q[req] + tok0;
+  const int* table = p.block_tables + (int64_t)req * p.table_width;
+
+  const int vs = blockIdx.y % x.v_splits;
+  const int hc = (blockIdx.y / x.v_splits) % x.head_chunks;
+  const int g = blockIdx.y / (x.v_splits * x.head_chunks);
+  const int group = p.heads / p.kv_heads;
+  const int h0 = hc * x.heads_per_wg;
+  const int nh_here = min(x.heads_per_wg, group - h0);
+  const int v0 = vs * VW;
+  const bool alias = p.v_plane == p.k_plane;
+
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(ra_smem);   // [RM_KT][KROW]
+  bf16_t* Vt = Ks + RM_KT * KROW;                    // [VW][VROW]
+  const bf16_t* q = (const bf16_t*)p.q;
+  const bf16_t* kc = (const bf16_t*)p.k_plane;
+  const bf16_t* vc = (const bf16_t*)p.v_plane;
+
+  // this wave's units: (head of the group, map)
+  int unit_head[UPW];
+  bool unit_ok[UPW];
+  ra_bf16x8_t qf[UPW][D32];
+  const int qi = min(l16, nq - 1);
+#pragma unroll
+  for (int a = 0; a < UPW; ++a) {
+    const int hl = MAPS == 2 ? wave : wave + 4 * a;
+    const int map = MAPS == 2 ? a : 0;
+    unit_ok[a] = hl < nh_here;
+    unit_head[a] = g * group + h0 + min(hl, nh_here - 1);
+    const bf16_t* qrow = q + (row0 + qi) * p.q_stride + (int64_t)unit_head[a] * p.q_head_stride + map * D + slot * 8;
+#pragma unroll
+    for (int ks = 0; ks < D32; ++ks) qf[a][ks] = ra_load8(qrow + ks * 32);
+  }
+
+  // this workgroup's run of the key chunks
+  const int n_chunks = (last - first) / RM_KT + 1;
+  const int runs = gridDim.z;
+  const int per_run = (n_chunks + runs - 1) / runs;
+  const int c_begin = blockIdx.z * per_run, c_end = min(n_chunks, c_begin + per_run);
+
+  uint4 kreg[PFK], vreg[PFV];
+  auto row_of = [&](int j) -> int64_t {
+    if (j > last) return -1;
+    const int b = j / p.block_size;
+    const int page = b < p.table_width ? table[b] : -1;
+    const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
+    return (page >= 0 && row < p.cache_rows) ? row : -1;
+  };
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int it = 0; it < PFK; ++it) {
+      const int idx = tid + it * 256;
+      const int at = min(idx, RM_KT * KPR - 1);
+      const int e = at % KPR, jj = at / KPR;
+      const int64_t row = row_of(k0 + jj);
+      const uint4 v = *reinterpret_cast<const uint4*>(kc + (row >= 0 ? row : 0) * p.k_row + (int64_t)g * DA + e * 8);
+      kreg[it] = (row >= 0 && idx == at) ? v : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int it = 0; it < PFV; ++it) {
+      const int idx = tid + it * 256;
+      const int at = min(idx, RM_KT * VPR - 1);
+      const int e = at % VPR, jj = at / VPR;
+      const int64_t row = row_of(k0 + jj);
+      const int64_t col = alias ? (int64_t)v0 : (int64_t)g * p.vdim + v0;
+      const uint4 v = *reinterpret_cast<const uint4*>(vc + (row >= 0 ? row : 0) * p.v_row + col + e * 8);
+      vreg[it] = (row >= 0 && idx == at) ? v : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store = [&]() {
+#pragma unroll
+    for (int it = 0; it < PFK; ++it) {
+      const int idx = tid + it * 256;
+      if (idx < RM_KT * KPR) {
+        const int e = idx % KPR, jj = idx / KPR;
+        *reinterpret_cast<uint4*>(Ks + jj * KROW + e * 8) = kreg[it];
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < PFV; ++it) {
+      const int idx = tid + it * 256;
+      if (idx < RM_KT * VPR) {
+        const int e = idx % VPR, jj = idx / VPR;
+        const uint32_t w[4] = {vreg[it].x, vreg[it].y, vreg[it].z, vreg[it].w};
+        uint16_t* dst = reinterpret_cast<uint16_t*>(Vt) + (e * 8) * VROW + jj;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          dst[(2 * u) * VROW] = (uint16_t)(w[u] & 0xffffu);
+          dst[(2 * u + 1) * VROW] = (uint16_t)(w[u] >> 16);
+        }
+      }
+    }
+  };
+
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float scale2 = p.scale * LOG2E;
+  float m[UPW], l[UPW];
+  ra_f32x4_t out[UPW][NT];
+#pragma unroll
+  for (int a = 0; a < UPW; ++a) {
+    // the sink counts once: in the first run of the keys
+    const bool sink_here = p.sink != nullptr && blockIdx.z == 0;
+    m[a] = sink_here ? p.sink[unit_head[a]] * LOG2E : -3.0e38f;
+    l[a] = (sink_here && slot == 0) ? 1.0f : 0.0f;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) out[a][nt] = ra_f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+
+  if (c_begin < c_end) fetch(first + c_begin * RM_KT);
+  for (int c = c_begin; c < c_end; ++c) {
+    const int k0 = first + c * RM_KT;
+    __syncthreads();
+    store();
+    if (c + 1 < c_end) fetch(k0 + RM_KT);
+    __syncthreads();
+    const bool inside = nq == 16 && k0 + RM_KT - 1 <= pos0 && k0 >= lo_last;
+    ra_bf16x8_t pw[UPW];
+#pragma unroll
+    for (int a = 0; a < UPW; ++a) {
+      const int map = MAPS == 2 ? a : 0;
+      ra_f32x4_t acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+      const bf16_t* kb = Ks + l16 * KROW + map * D + slot * 8;
+#pragma unroll
+      for (int ks = 0; ks < D32; ++ks) {
+        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ra_load8(kb + ks * 32), qf[a][ks], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ra_load8(kb + 16 * KROW + ks * 32), qf[a][ks], acc1, 0, 0, 0);
+      }
+      const int pos = pos0 + l16;
+      const int lo = ra_oldest_seen(p.mask_kind, p.mask_size, pos);
+      float s[8];
+      float top = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int j = k0 + (u >> 2) * 16 + slot * 4 + (u & 3);
+        float v = (u < 4 ? acc0[u & 3] : acc1[u & 3]) * scale2;
+        if (!inside) v = (l16 < nq && j <= pos && j >= lo) ? v : -INFINITY;
+        s[u] = v;
+        top = fmaxf(top, v);
+      }
+      top = cw_quad_max(top);
+      const float mn = fmaxf(m[a], top);
+      const float alpha = __builtin_amdgcn_exp2f(m[a] - mn);
+      m[a] = mn;
+      float sum = 0.0f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float w = __builtin_amdgcn_exp2f(s[u] - mn);
+        sum += w;
+        pw[a][u] = (__bf16)w;
+      }
+      l[a] = l[a] * alpha + sum;
+      // the accumulators' rows are queries slot * 4 + e: each takes its own query's factor
+      if (__ballot(alpha != 1.0f) != 0) {
+        float ar[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ar[e] = __shfl(alpha, slot * 4 + e, 64);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[a][nt][e] *= ar[e];
+      }
+    }
+    // values: a fragment (16 value columns, 32 keys) serves all of the wave's units
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const bf16_t* vb = Vt + (nt * 16 + l16) * VROW + slot * 4;
+      const uint2 lo4 = *reinterpret_cast<const uint2*>(vb), hi4 = *reinterpret_cast<const uint2*>(vb + 16);
+      const uint4 both = make_uint4(lo4.x, lo4.y, hi4.x, hi4.y);
+      const ra_bf16x8_t vf = *reinterpret_cast<const ra_bf16x8_t*>(&both);
+#pragma unroll
+      for (int a = 0; a < UPW; ++a) out[a][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pw[a], vf, out[a][nt], 0, 0, 0);
+    }
+  }
+
+  if (runs > 1) {
+    // maximum, denominator and unnormalised sums of this run, per unit and query
+    const int64_t wg = ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * runs + blockIdx.z;
+    float* base = x.workspace + wg * (4 * UPW * 16 * (2 + VW));
+#pragma unroll
+    for (int a = 0; a < UPW; ++a) {
+      const float total = cw_quad_sum(l[a]);
+      float* u = base + (int64_t)(wave * UPW + a) * 16 * (2 + VW);
+      if (slot == 0) { u[l16 * (2 + VW)] = m[a]; u[l16 * (2 + VW) + 1] = total; }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) u[(slot * 4 + e) * (2 + VW) + 2 + nt * 16 + l16] = out[a][nt][e];
+    }
+    return;
+  }
+
+  // ---- finish: denominators, the two maps' difference, the head norm
+  float inv_row[UPW][4];
+#pragma unroll
+  for (int a = 0; a < UPW; ++a) {
+    const float total = cw_quad_sum(l[a]);
+    const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) inv_row[a][e] = __shfl(inv, slot * 4 + e, 64);
+  }
+  const float lam = (MAPS == 2 && p.lambda) ? p.lambda[0] : 0.0f;
+  constexpr int OUTS = MAPS == 2 ? 1 : UPW;
+  bf16_t* o = (bf16_t*)p.out;
+#pragma unroll
+  for (int a = 0; a < OUTS; ++a) {
+    float sq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float v = out[a][nt][e] * inv_row[a][e];
+        if (MAPS == 2) v -= lam * out[UPW - 1][nt][e] * inv_row[UPW - 1][e];
+        out[a][nt][e] = v;
+        sq[e] += v * v;
+      }
+    float mult[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    if (p.head_norm) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) sq[e] += __shfl_xor(sq[e], off, 64);
+        mult[e] = p.post_mult / sqrtf(sq[e] / (float)p.vdim + p.norm_eps);
+      }
+    }
+    if (unit_ok[a]) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = slot * 4 + e;
+          if (i < nq)
+            o[(row0 + i) * p.out_stride + (int64_t)unit_head[a] * p.out_head_stride + v0 + nt * 16 + l16] =
+                __float2bfloat16(out[a][nt][e] * mult[e]);
+        }
+    }
+  }
+}
+
+// Puts the runs of rows_mfma_kernel together: one workgroup per (item, key/value head, head chunk,
+// value split); a thread takes one query (tid / 16) and the value columns tid % 16 + 16 i.
+template <int MAPS>
+__global__ __launch_bounds__(256) void rows_merge_kernel(const RowsAttnParams p, const RowsMfmaExtra x, int runs, int upw,
+                                                         int vw) {
+  const int tid = threadIdx.x, qi = tid >> 4, sub = tid & 15;
+  const int* item = p.items + 4 * (int64_t)blockIdx.x;
+  const int req = item[0], tok0 = item[1];
+  const int q_len = p.cu_q[req + 1] - p.cu_q[req];
+  if (tok0 >= q_len) return;
+  const int nq = min(min(item[2], 16), q_len - tok0);
+  const int64_t row0 = (int64_t)p.cu_q[req] + tok0;
+  const int vs = blockIdx.y % x.v_splits;
+  const int hc = (blockIdx.y / x.v_splits) % x.head_chunks;
+  const int g = blockIdx.y / (x.v_splits * x.head_chunks);
+  const int group = p.heads / p.kv_heads;
+  const int h0 = hc * x.heads_per_wg;
+  const int nh_here = min(x.heads_per_wg, group - h0);
+  const int v0 = vs * vw;
+  const int stride_q = 2 + vw, stride_unit = 16 * stride_q, stride_run = 4 * upw * stride_unit;
+  const float* base = x.workspace + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * runs * stride_run;
+  const float lam = (MAPS == 2 && p.lambda) ? p.lambda[0] : 0.0f;
+  bf16_t* o = (bf16_t*)p.out;
+  for (int hl = 0; hl < nh_here; ++hl) {
+    float val[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) val[i] = 0.0f;
+#pragma unroll
+    for (int map = 0; map < MAPS; ++map) {
+      // the unit's place in a run's block: (wave, a)
+      const int unit = MAPS == 2 ? hl * upw + map : (hl % 4) * upw + hl / 4;
+      const float* u = base + (int64_t)unit * stride_unit + qi * stride_q;
+      float top = -3.0e38f;
+      for (int r = 0; r < runs; ++r) top = fmaxf(top, u[(int64_t)r * stride_run]);
+      float den = 0.0f;
+      float part[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) part[i] = 0.0f;
+      for (int r = 0; r < runs; ++r) {
+        const float* ur = u + (int64_t)r * stride_run;
+        const float f = __builtin_amdgcn_exp2f(ur[0] - top);
+        den += ur[1] * f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (sub + 16 * i < vw) part[i] += ur[2 + sub + 16 * i] * f;
+      }
+      const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) val[i] += (map == 0 ? 1.0f : -lam) * part[i] * inv;
+    }
+    float mult = 1.0f;
+    if (p.head_norm) {
+      float sq = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (sub + 16 * i < vw) sq += val[i] * val[i];
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+      mult = p.post_mult / sqrtf(sq / (float)p.vdim + p.norm_eps);
+    }
+    if (qi < nq) {
+      const int head = g * group + h0 + hl;
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (sub + 16 * i < vw)
+          o[(row0 + qi) * p.out_stride + (int64_t)head * p.out_head_stride + v0 + sub + 16 * i] = __float2bfloat16(val[i] * mult);
+    }
+  }
+}
+
+// How the matrix-core kernel cuts a geometry: value columns a workgroup takes (16 * nt), how many
+// workgroups share the columns, units a wave holds; 0 in *nt: not taken. Key rows of 32 * d32
+// elements a map for d32 in {2, 4} (two maps) or {5, 10, 18} (one map), value rows of 64, 128 or 256
+// (two maps: the head norm needs all columns in one workgroup) or 128, 256, 512 (one map).
+static void ra_mfma_shape(int maps, int dim, int vdim, int* d32, int* nt, int* v_splits, int* upw) {
+  *nt = 0; *v_splits = 1; *upw = maps == 2 ? 2 : 1; *d32 = dim / 32;
+  if (dim % 32) return;
+  if (maps == 2) {
+    if (*d32 != 2 && *d32 != 4) return;
+    if (vdim == 64) *nt = 4; else if (vdim == 128) *nt = 8; else if (vdim == 256) *nt = 16;
+  } else {
+    if (*d32 != 5 && *d32 != 10 && *d32 != 18) return;
+    if (vdim == 128) *nt = 8; else if (vdim == 256) *nt = 16; else if (vdim == 512) { *nt = 16; *v_splits = 2; }
+  }
+}
+
+CW_EXPORT int cw_rows_mfma_supported(int maps, int dim, int vdim) {
+  int d32, nt, vsp, upw;
+  ra_mfma_shape(maps, dim, vdim, &d32, &nt, &vsp, &upw);
+  return nt != 0;
+}
+
+// Workgroups of one run of keys: (items, y); and the floats of workspace that ``runs`` runs need.
+CW_EXPORT int cw_rows_mfma_grid_y(int heads, int kv_heads, int maps, int dim, int vdim) {
+  int d32, nt, vsp, upw;
+  ra_mfma_shape(maps, dim, vdim, &d32, &nt, &vsp, &upw);
+  if (!nt || heads % kv_heads) return 0;
+  const int per_wg = maps == 2 ? 4 : 4 * upw, group = heads / kv_heads;
+  return kv_heads * ((group + per_wg - 1) / per_wg) * vsp;
+}
+CW_EXPORT int64_t cw_rows_mfma_workspace_floats(int n_items, int heads, int kv_heads, int maps, int dim, int vdim, int runs) {
+  int d32, nt, vsp, upw;
+  ra_mfma_shape(maps, dim, vdim, &d32, &nt, &vsp, &upw);
+  if (!nt || runs <= 1) return 0;
+  return (int64_t)n_items * cw_rows_mfma_grid_y(heads, kv_heads, maps, dim, vdim) * runs * 4 * upw * 16 * (2 + 16 * nt);
+}
+
+CW_EXPORT int cw_rows_attention_mfma(const void* q, int64_t q_stride, int64_t q_head_stride, void* out, int64_t out_stride,
+                                     int64_t out_head_stride, const void* k_plane, const void* v_plane, int k_row, int v_row,
+                                     int64_t cache_rows, const int* block_tables, int table_width, const int* ctx_lens,
+                                     const int* cu_q, const int* items, int n_items, const float* sink, const float* lambda,
+                                     int heads, int kv_heads, int dim, int vdim, int maps, int block_size, int mask_kind,
+                                     int mask_size, float scale, int head_norm, float norm_eps, float post_mult, int runs,
+                                     float* workspace, int64_t workspace_floats, hipStream_t stream) {
+  if (n_items < 0 || !q || !out || !k_plane || !v_plane || !block_tables || !ctx_lens || !cu_q || !items) return CW_ERR_ARG;
+  if (block_size <= 0 || table_width <= 0 || mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && mask_size < 1)) return CW_ERR_ARG;
+  if ((maps == 2 && !lambda) || runs < 1 || runs > 64) return CW_ERR_ARG;
+  int d32, nt, vsp, upw;
+  ra_mfma_shape(maps, dim, vdim, &d32, &nt, &vsp, &upw);
+  if (!nt || heads % kv_heads) return CW_ERR_SIZE;
+  const int alias = v_plane == k_plane;
+  if (alias && (maps != 1 || kv_heads != 1 || vdim > dim)) return CW_ERR_ARG;
+  if (head_norm && vsp != 1) return CW_ERR_ARG;
+  // 16-byte loads: rows and heads begin at multiples of 8 elements
+  if (q_stride % 8 || q_head_stride % 8 || k_row % 8 || (!alias && v_row % 8) || ((uintptr_t)q | (uintptr_t)k_plane | (uintptr_t)v_plane) % 16)
+    return CW_ERR_ARG;
+  if (k_row < kv_heads * maps * dim || (!alias && v_row < kv_heads * vdim)) return CW_ERR_ARG;
+  if (runs > 1 && (!workspace || workspace_floats < cw_rows_mfma_workspace_floats(n_items, heads, kv_heads, maps, dim, vdim, runs)))
+    return CW_ERR_ARG;
+  if (n_items == 0) return CW_OK;
+  RowsAttnParams p;
+  p.q = q; p.q_stride = q_stride; p.q_head_stride = q_head_stride; p.out = out; p.out_stride = out_stride;
+  p.out_head_stride = out_head_stride; p.k_plane = k_plane; p.v_plane = v_plane; p.k_row = k_row;
+  p.v_row = alias ? k_row : v_row; p.cache_rows = cache_rows; p.block_tables = block_tables; p.table_width = table_width;
+  p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items; p.sink = sink; p.lambda = lambda; p.heads = heads;
+  p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.maps = maps; p.heads_per_group = 0; p.tokens_per_item = 16;
+  p.key_chunk = RM_KT; p.block_size = block_size; p.mask_kind = mask_kind; p.mask_size = mask_size; p.scale = scale;
+  p.head_norm = head_norm; p.norm_eps = norm_eps; p.post_mult = post_mult;
+  RowsMfmaExtra x;
+  x.workspace = workspace; x.v_splits = vsp; x.heads_per_wg = maps == 2 ? 4 : 4 * upw;
+  const int group = heads / kv_heads;
+  x.head_chunks = (group + x.heads_per_wg - 1) / x.heads_per_wg;
+  dim3 grid(n_items, kv_heads * x.head_chunks * vsp, runs), block(256);
+  const size_t smem = ((size_t)RM_KT * (maps * dim + 8) + (size_t)16 * nt * (RM_KT + 8)) * 2;
+#define CW_LAUNCH(D32_, NT_, UPW_, MAPS_)                                                                          \
+  do {                                                                                                             \
+    if (smem > 48 * 1024 && hipFuncSetAttribute((const void*)rows_mfma_kernel<D32_, NT_, UPW_, MAPS_>,             \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) \
+      return CW_ERR_LAUNCH;                                                                                        \
+    hipLaunchKernelGGL((rows_mfma_kernel<D32_, NT_, UPW_, MAPS_>), grid, block, smem, stream, p, x);               \
+  } while (0)
+#define CW_PICK_NT(D32_, UPW_, MAPS_, A_, B_, C_)                                                                  \
+  do {                                                                                                             \
+    if (nt == A_) CW_LAUNCH(D32_, A_, UPW_, MAPS_);                                                                \
+    else if (nt == B_) CW_LAUNCH(D32_, B_, UPW_, MAPS_);                                                           \
+    else CW_LAUNCH(D32_, C_, UPW_, MAPS_);                                                                         \
+  } while (0)
+  if (maps == 2) {
+    if (d32 == 2) CW_PICK_NT(2, 2, 2, 4, 8, 16);
+    else CW_PICK_NT(4, 2, 2, 4, 8, 16);
+  } else {
+    if (d32 == 5) CW_PICK_NT(5, 1, 1, 8, 16, 16);
+    else if (d32 == 10) CW_PICK_NT(10, 1, 1, 8, 16, 16);
+    else CW_PICK_NT(18, 1, 1, 8, 16, 16);
+  }
+#undef CW_PICK_NT
+#undef CW_LAUNCH
+  if (hipGetLastError() != hipSuccess) return CW_ERR_LAUNCH;
+  if (runs > 1) {
+    dim3 mgrid(n_items, grid.y);
+    if (maps == 2) hipLaunchKernelGGL(rows_merge_kernel<2>, mgrid, block, 0, stream, p, x, runs, upw, 16 * nt);
+    else hipLaunchKernelGGL(rows_merge_kernel<1>, mgrid, block, 0, stream, p, x, runs, upw, 16 * nt);
+  }
+  return cw_launch_status();
+}

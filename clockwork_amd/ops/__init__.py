@@ -137,6 +137,11 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_rows_attention_key_chunk": [I, I, I, I],
             "cw_rows_attention_heads_per_group": [I, I, I],
             "cw_rows_attention_tokens_per_item": [I, I, I],
+            "cw_rows_mfma_supported": [I, I, I],
+            "cw_rows_mfma_grid_y": [I, I, I, I, I],
+            "cw_rows_mfma_workspace_floats": [I, I, I, I, I, I, I],
+            "cw_rows_attention_mfma": [P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F,
+                                       I, P, L, P],
             "cw_rows_attention": [I, P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F, P],
         },
         "sink_attention": {
@@ -1685,6 +1690,27 @@ def rows_attention_tokens_per_item(heads: int, kv_heads: int, maps: int = 1) -> 
     return int(_load("rows_attention").cw_rows_attention_tokens_per_item(heads, kv_heads, maps))
 
 
+ROWS_MFMA_TOKENS = 16   # tokens of one request that a work item of the matrix-core kernel holds
+
+
+def rows_mfma_supported(dim: int, vdim: int, maps: int, dtype) -> bool:
+    """Does the matrix-core kernel take this geometry? bfloat16; key rows of 64 or 128 elements a
+    map with value rows of 64, 128 or 256 (two maps), key rows of 160, 320 or 576 with value rows
+    of 128, 256 or 512 (one map)."""
+    return dtype == torch.bfloat16 and bool(_load("rows_attention").cw_rows_mfma_supported(maps, dim, vdim))
+
+
+def rows_mfma_key_runs(n_items: int, longest: int, heads: int, kv_heads: int, dim: int, vdim: int, maps: int,
+                       compute_units: int) -> int:
+    """Into how many runs the matrix-core kernel cuts every item's keys: as many as there are idle
+    compute units for while the longest key range gives each run 128 keys, 64 at most (a step of
+    single tokens, or a short portion behind a long context, would leave most of the card idle)."""
+    per_run = n_items * int(_load("rows_attention").cw_rows_mfma_grid_y(heads, kv_heads, maps, dim, vdim))
+    if per_run <= 0:
+        return 1
+    return int(max(1, min(compute_units // per_run, longest // 128, 64)))
+
+
 def heads_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[h] = x[h] @ weight[h].T for every head: ``x`` [heads, T, n_in], ``weight``
     [heads, n_out, n_in], ``out`` [heads, T, n_out]; x and out may be views whose rows lie apart
@@ -1702,7 +1728,7 @@ def heads_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> to
 def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_tables, ctx_lens, cu_q, items, n_items: int,
                    heads: int, kv_heads: int, dim: int, vdim: int, block_size: int, scale: float, maps: int = 1,
                    mask: str = "causal", mask_size: int = 0, sink=None, lam=None, head_norm_eps=None,
-                   post_mult: float = 1.0) -> None:
+                   post_mult: float = 1.0, mfma: bool = False, key_runs: int = 1) -> None:
     """Softmax attention of the step's queries over paged rows. Query (t, head, map, d) lies at
     ``q.flatten()[t * q_strides[0] + head * q_strides[1] + map * dim + d]``, output (t, head, c) at
     ``out.flatten()[t * out_strides[0] + head * out_strides[1] + c]`` (token-major or head-major
@@ -1715,7 +1741,9 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
     map 0 minus ``lam`` (one float32 element) times map 1. ``head_norm_eps`` not None: the head's
     output is divided by its root mean square and multiplied by ``post_mult``. ``items`` int32
     [n_items, 4]: (request, first token, tokens, 0) with at most
-    ``rows_attention_tokens_per_item`` tokens each."""
+    ``rows_attention_tokens_per_item`` tokens each. ``mfma``: the matrix-core kernel
+    (``rows_mfma_supported``; items of up to ``ROWS_MFMA_TOKENS`` tokens), every item's keys cut
+    into ``key_runs`` runs that a second kernel puts together."""
     alias = v_plane is None
     _gpu(q, out, k_plane, v_plane, block_tables, ctx_lens, cu_q, items, sink, lam)
     qs, qh = int(q_strides[0]), int(q_strides[1])
@@ -1746,6 +1774,18 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
     _need((maps == 1 and lam is None) or (maps == 2 and lam is not None and lam.dtype == torch.float32 and lam.numel() == 1),
           "two maps take one float32 lambda, one map none")
     _need(mask in MASK_KINDS and (mask == "causal" or mask_size >= 1), f"mask {mask!r} of size {mask_size}")
+    if mfma:
+        lib = _load("rows_attention")
+        _need(rows_mfma_supported(dim, vdim, maps, q.dtype), "the matrix-core kernel does not take this geometry")
+        need = int(lib.cw_rows_mfma_workspace_floats(n_items, heads, kv_heads, maps, dim, vdim, key_runs))
+        workspace = torch.empty(need, dtype=torch.float32, device=q.device) if need else None
+        _check(lib.cw_rows_attention_mfma(
+            _ptr(q), qs, qh, _ptr(out), os_, oh, _ptr(k_plane), _ptr(k_plane if alias else v_plane), k2.shape[1], v_row, rows,
+            _ptr(block_tables), block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(sink), _ptr(lam),
+            heads, kv_heads, dim, vdim, maps, block_size, MASK_KINDS[mask], int(mask_size), float(scale),
+            0 if head_norm_eps is None else 1, float(head_norm_eps or 0.0), float(post_mult), int(key_runs), _ptr(workspace), need,
+            _stream()), "rows_attention_mfma")
+        return
     _check(_load("rows_attention").cw_rows_attention(
         dtype_code(q.dtype), _ptr(q), qs, qh, _ptr(out), os_, oh, _ptr(k_plane), _ptr(k_plane if alias else v_plane), k2.shape[1],
         v_row, rows, _ptr(block_tables), block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(sink),

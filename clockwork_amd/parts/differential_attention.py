@@ -15,7 +15,7 @@ import torch
 from clockwork_amd import ops
 from clockwork_amd.config.spec import PagedRowsSpec, ParamSpec
 from clockwork_amd.parts.base import EntryCache, Part
-from clockwork_amd.parts.sink_attention import query_runs
+from clockwork_amd.parts.sink_attention import longest_key_range, query_runs
 from clockwork_amd.parts.specs import DifferentialAttentionSpec
 
 MAPS = 2
@@ -69,10 +69,27 @@ class DifferentialAttention(Part):
         if not ops.rows_attention_supported(s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim, maps=MAPS):
             raise ValueError(f"two-map attention with keys of {s.key_dim} and values of {s.value_dim} elements is beyond "
                              "the attention kernel for paged rows (value_dim up to 512, tiles of 150 KB of LDS)")
-        self.run = ops.rows_attention_tokens_per_item(s.num_heads, s.num_kv_heads, MAPS)
+        # bfloat16 with the common head sizes runs on the matrix cores (16-byte loads: rows begin at multiples of 8)
+        self.mfma = (ops.rows_mfma_supported(s.key_dim, s.value_dim, MAPS, dtype)
+                     and (self.q_width + self.k_width + self.v_width) % 8 == 0)
+        self.run = ops.ROWS_MFMA_TOKENS if self.mfma else ops.rows_attention_tokens_per_item(s.num_heads, s.num_kv_heads, MAPS)
+
+    def _plan(self, ctx):
+        """(work items, their number, runs that every item's keys are cut into)."""
+        s = self.spec
+        key = ("two-map attention", s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim, s.segment, s.window, self.mfma)
+        plan = ctx.plans.get(key)
+        if plan is None:
+            items, n_items = query_runs(ctx, self.run)
+            runs = 1
+            if self.mfma:
+                runs = ops.rows_mfma_key_runs(n_items, longest_key_range(ctx, s.window, s.segment), s.num_heads, s.num_kv_heads,
+                                              s.key_dim, s.value_dim, MAPS, ctx.num_compute_units)
+            plan = ctx.plans[key] = (items, n_items, runs)
+        return plan
 
     def prepare(self, ctx) -> None:
-        query_runs(ctx, self.run)
+        self._plan(ctx)
 
     def forward(self, x: torch.Tensor, ctx, cache: EntryCache) -> torch.Tensor:
         s = self.spec
@@ -84,10 +101,10 @@ class DifferentialAttention(Part):
         ops.bias_store(qkv, 0, self.q_width, self.q_width + self.k_width, self.q_width, self.k_width, self.v_width,
                        self.qkv_bias, ctx.slots[cache.group], k_plane, v_plane)
         out = torch.empty((x.shape[0], s.num_heads * s.value_dim), dtype=x.dtype, device=x.device)
-        items, n_items = query_runs(ctx, self.run)
+        items, n_items, runs = self._plan(ctx)
         kind, size = self.mask()
         ops.rows_attention(qkv, (qkv.shape[1], MAPS * s.key_dim), out, (out.shape[1], s.value_dim), k_plane, v_plane,
                            ctx.block_tables[cache.group], ctx.ctx_lens, ctx.cu_q, items, n_items, s.num_heads, s.num_kv_heads,
                            s.key_dim, s.value_dim, cache.block_size, s.scale, maps=MAPS, mask=kind, mask_size=size, lam=self.lam,
-                           head_norm_eps=s.norm_eps, post_mult=1.0 - s.lambda_init)
+                           head_norm_eps=s.norm_eps, post_mult=1.0 - s.lambda_init, mfma=self.mfma, key_runs=runs)
         return ops.linear(out, self.out_weight, policy=policy)

@@ -21,7 +21,7 @@ import torch
 from clockwork_amd import ops
 from clockwork_amd.config.spec import PagedRowsSpec, ParamSpec
 from clockwork_amd.parts.base import EntryCache, Part
-from clockwork_amd.parts.sink_attention import query_runs
+from clockwork_amd.parts.sink_attention import longest_key_range, query_runs
 from clockwork_amd.parts.specs import LatentAttentionSpec
 
 
@@ -74,10 +74,26 @@ class LatentAttention(Part):
         if not ops.rows_attention_supported(s.num_heads, 1, self.row, s.kv_rank, alias=True):
             raise ValueError(f"latent attention with rows of {self.row} elements is beyond the attention kernel for paged rows "
                              "(a latent of up to 512 elements, tiles of 150 KB of LDS)")
-        self.run = ops.rows_attention_tokens_per_item(s.num_heads, 1, 1)
+        # bfloat16 with the common latent sizes runs on the matrix cores
+        self.mfma = ops.rows_mfma_supported(self.row, s.kv_rank, 1, dtype)
+        self.run = ops.ROWS_MFMA_TOKENS if self.mfma else ops.rows_attention_tokens_per_item(s.num_heads, 1, 1)
+
+    def _plan(self, ctx):
+        """(work items, their number, runs that every item's keys are cut into)."""
+        s = self.spec
+        key = ("latent attention", s.num_heads, self.row, s.kv_rank, s.window, self.mfma)
+        plan = ctx.plans.get(key)
+        if plan is None:
+            items, n_items = query_runs(ctx, self.run)
+            runs = 1
+            if self.mfma:
+                runs = ops.rows_mfma_key_runs(n_items, longest_key_range(ctx, s.window), s.num_heads, 1, self.row, s.kv_rank, 1,
+                                              ctx.num_compute_units)
+            plan = ctx.plans[key] = (items, n_items, runs)
+        return plan
 
     def prepare(self, ctx) -> None:
-        query_runs(ctx, self.run)
+        self._plan(ctx)
 
     def forward(self, x: torch.Tensor, ctx, cache: EntryCache) -> torch.Tensor:
         s = self.spec
@@ -98,11 +114,11 @@ class LatentAttention(Part):
             ops.rotate_part(q, (q.shape[1], self.q_head), s.key_dim, qa, (self.row, T * self.row), s.kv_rank, H, s.rope_dim,
                             s.rotary_dims, ctx.positions, self.freq)
         ol = torch.empty((H, T, s.kv_rank), dtype=x.dtype, device=x.device)
-        items, n_items = query_runs(ctx, self.run)
+        items, n_items, runs = self._plan(ctx)
         kind, size = ("window", s.window) if s.window is not None else ("causal", 0)
         ops.rows_attention(qa, (self.row, T * self.row), ol, (s.kv_rank, T * s.kv_rank), plane, None,
                            ctx.block_tables[cache.group], ctx.ctx_lens, ctx.cu_q, items, n_items, H, 1, self.row, s.kv_rank,
-                           cache.block_size, s.scale, mask=kind, mask_size=size, sink=self.sink)
+                           cache.block_size, s.scale, mask=kind, mask_size=size, sink=self.sink, mfma=self.mfma, key_runs=runs)
         out = torch.empty((T, self.o_width), dtype=x.dtype, device=x.device)
         ops.heads_linear(ol, self.v_up, out.view(T, H, s.value_dim).transpose(0, 1))
         if s.output_gate:

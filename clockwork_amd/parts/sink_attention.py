@@ -45,6 +45,16 @@ def query_runs(ctx, run: int, skip_single: bool = False):
     return plan
 
 
+def longest_key_range(ctx, window=None, segment=None) -> int:
+    """The most keys that a token of this step reads: its request's length, capped by a window or
+    by the segment's size."""
+    longest = max(ctx.h_ctx_lens, default=0)
+    for cap in (window, segment):
+        if cap is not None:
+            longest = min(longest, cap)
+    return longest
+
+
 class SinkAttention(Part):
     graph_safe = True
 

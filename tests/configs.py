@@ -186,16 +186,16 @@ PESORAX_C = {
         _pesorax_attention(1, 1, 32, 8, 0.18, 0.6, 17, 24),
     ],
 }
-# layers of unlike sizes for long requests: segments of 77 to 1500, a latent of 256 + 64 elements,
-# sizes that the matrix cores take and sizes that they do not
+# layers of unlike sizes for long requests: segments of 77 to 1500, latents of 256 + 64 and 128 + 32
+# elements, sizes that the matrix cores take (layers 1 to 4) and one that they do not
 PESORAX_LONG = {
     "architecture": "Pesorax", "vocab": 211, "width": 192, "residual_mult": 0.4, "norm": {"eps": 2e-6},
     "loop": {"start": 0, "stop": 1, "times": 2},
     "layers": [
         _pesorax_attention(6, 3, 32, 48, 0.3, 0.4, 200, 384),
-        _pesorax_latent(8, 64, 32, 32, 64, 96, 256, 0.2, 10000.0, None),
+        _pesorax_latent(8, 64, 64, 32, 64, 96, 256, 0.2, 10000.0, None),
         _pesorax_attention(8, 2, 64, 128, 0.15, 0.7, 1500, 100),
-        _pesorax_latent(16, 32, 64, 32, 32, 64, 128, 0.25, 500.0, 64),
+        _pesorax_latent(16, 32, 32, 32, 32, 64, 128, 0.25, 500.0, 64),
         _pesorax_attention(4, 4, 64, 64, 0.2, 0.2, 77, None),
     ],
 }

@@ -108,6 +108,42 @@ def test_two_map_attention_whole_in_portions_and_token_by_token(dtype, shape):
     for cuts in ([T], [5, 1, 1, 17, 2, 1, 2, 32], [1] * T):
         got = _step_through(part, part.cache_need(), x, cuts, dtype)
         close(got, want, dtype)
+    _matrix_cores_against_plain_arithmetic(part, x, want, dtype)
+
+
+def _matrix_cores_against_plain_arithmetic(part, x, want, dtype):
+    """Where the matrix-core kernel runs: against the plain-arithmetic kernel on the very same
+    bfloat16 queries, keys and values. They differ by the order of their sums, by the weights'
+    rounding to bfloat16 before the value product and by the rounding of the output, a fraction of
+    what separates either from the float64 result."""
+    if not part.mfma:
+        return
+    assert dtype == torch.bfloat16
+    T = x.shape[0]
+    fast = _step_through(part, part.cache_need(), x, [T], dtype)
+    s = part.spec
+    part.mfma = False
+    part.run = (ops.rows_attention_tokens_per_item(s.num_heads, s.num_kv_heads, 2) if hasattr(s, "num_kv_heads")
+                else ops.rows_attention_tokens_per_item(s.num_heads, 1, 1))
+    slow = _step_through(part, part.cache_need(), x, [T], dtype)
+    scale = float(want.square().mean().sqrt())
+    assert float((fast - slow).abs().max()) < 3e-2 * scale and float((fast - slow).square().mean().sqrt()) < 6e-3 * scale
+
+
+def test_the_matrix_core_kernel_is_the_one_that_runs_for_bfloat16():
+    two = DifferentialAttentionSpec(hidden_size=64, num_heads=8, num_kv_heads=2, key_dim=64, value_dim=128, scale=0.1,
+                                    lambda_init=0.5, norm_eps=1e-6, segment=40)
+    latent = LatentAttentionSpec(hidden_size=64, num_heads=4, key_dim=32, rope_dim=64, value_dim=32, q_rank=48, kv_rank=256,
+                                 scale=0.1, rope_base=100.0, rotary_dims=64, norm_eps=1e-6)
+    for spec in (two, latent):
+        for dtype, expected in ((torch.bfloat16, True), (torch.float32, False)):
+            part = build_part(spec)
+            bind(part, dtype)
+            assert part.mfma is expected and part.run == (16 if expected else part.run)
+    odd = build_part(DifferentialAttentionSpec(hidden_size=64, num_heads=4, num_kv_heads=2, key_dim=24, value_dim=16, scale=0.1,
+                                               lambda_init=0.5, norm_eps=1e-6, segment=9))
+    bind(odd, torch.bfloat16)
+    assert not odd.mfma and odd.run >= 1
 
 
 def test_two_map_attention_options_each_matter():
@@ -196,6 +232,7 @@ def test_a_far_key_among_hundreds_decides_the_two_map_output(dtype):
     segment sees, and gone at the first token of the next segment."""
     hidden, dim, vdim, segment = 32, 64, 64, 400
     spec, part, w = _loud_two_map_part(hidden, dim, vdim, segment, dtype)
+    assert part.mfma == (dtype == torch.bfloat16)
     T, loud = 850, 402
     x = torch.zeros(T, hidden)
     x[:, 1] = 1.0
@@ -242,6 +279,7 @@ def test_latent_attention_whole_in_portions_and_token_by_token(dtype, shape):
     for cuts in ([T], [5, 1, 1, 17, 2, 1, 2, 32], [1] * T):
         got = _step_through(part, part.cache_need(), x, cuts, dtype)
         close(got, want, dtype)
+    _matrix_cores_against_plain_arithmetic(part, x, want, dtype)
 
 
 def test_latent_attention_options_each_matter():
@@ -267,10 +305,11 @@ def test_sharp_latent_attention_over_hundreds_of_keys(dtype):
     """A scale so large that every query gives nearly all its weight to the one or two keys that
     fit it best, wherever among up to 500 earlier tokens they lie: a key that is lost or taken from
     a wrong page changes the output wholly. Positions enter through the rotated part alone."""
-    spec = LatentAttentionSpec(hidden_size=64, num_heads=4, key_dim=32, rope_dim=32, value_dim=32, q_rank=48, kv_rank=64,
-                               scale=2.5, rope_base=10000.0, rotary_dims=32, norm_eps=1e-6)
+    spec = LatentAttentionSpec(hidden_size=64, num_heads=6, key_dim=32, rope_dim=32, value_dim=32, q_rank=48, kv_rank=128,
+                               scale=1.2, rope_base=10000.0, rotary_dims=32, norm_eps=1e-6)
     part = build_part(spec)
     w = bind(part, dtype, seed=11, matrix_std=0.25, change=lambda v: v["sink"].fill_(-5.0))
+    assert part.mfma == (dtype == torch.bfloat16)   # in bfloat16 on the matrix cores, the keys of long ranges cut into runs
     T = 500
     x = torch.randn(T, 64, generator=torch.Generator().manual_seed(6)).to(dtype)
     want = plain.latent_attention(x.double(), _latent_names(w, spec), "", _latent_sizes(spec), 1e-6)
@@ -363,6 +402,8 @@ def test_long_requests_through_layers_of_unlike_sizes(tmp_path, dtype):
     ref = {rid: oracle.logits(toks) for rid, toks in requests.items()}
     for mode in ("whole", "prefill_then_decode", "portions", "mixed"):
         runner = replay.make_runner(model_dir, dtype, 16, 120, max_model_len=1600)
+        if dtype == "bfloat16":
+            assert [m.mfma for m in runner.model.mixers()] == [False, True, True, True, True]
         steps = replay.portions(requests, sizes=[2, 300, 7, 64, 129, 33, 512]) if mode == "portions" else getattr(replay, mode)(requests)
         _check(replay.run_trace(runner, steps), ref, dtype)
         assert all(p.num_free == runner.manager.num_blocks for p in runner.manager.pools)
