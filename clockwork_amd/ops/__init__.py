@@ -1715,13 +1715,25 @@ def heads_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> to
     """out[h] = x[h] @ weight[h].T for every head: ``x`` [heads, T, n_in], ``weight``
     [heads, n_out, n_in], ``out`` [heads, T, n_out]; x and out may be views whose rows lie apart
     (a slice of each head's columns), their last dimension dense. The library's batched product,
-    float32 accumulation (full float32 for float32 operands)."""
+    float32 accumulation (full float32 for float32 operands), always with the library's default
+    kernel: its tuner times candidates on copies of the operands that it sizes as
+    max(batch stride, rows * columns) * batch elements, which a slice of wider rows outgrows (rows
+    lie a whole token apart, heads a few columns), so a tuning run would read past its copy."""
     _need(x.dim() == 3 and weight.dim() == 3 and out.dim() == 3 and x.shape[0] == weight.shape[0] == out.shape[0]
           and x.shape[2] == weight.shape[2] and out.shape[2] == weight.shape[1] and x.shape[1] == out.shape[1],
           "heads_linear shapes")
     _need(x.dtype == weight.dtype == out.dtype and x.stride(2) == 1 and out.stride(2) == 1, "heads_linear types and strides")
     if x.shape[1]:
-        torch.bmm(x, weight.transpose(1, 2), out=out)
+        import torch.cuda.tunable as tunable
+
+        tuning = tunable.is_enabled() and tunable.tuning_is_enabled()
+        if tuning:
+            tunable.tuning_enable(False)
+        try:
+            torch.bmm(x, weight.transpose(1, 2), out=out)
+        finally:
+            if tuning:
+                tunable.tuning_enable(True)
     return out
 
 
