@@ -319,6 +319,8 @@ CW_EXPORT int cw_rows_attention(int dtype, const void* q, int64_t q_stride, int6
 // ======================================================================================
 typedef __attribute__((ext_vector_type(8))) __bf16 ra_bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float ra_f32x4_t;
+typedef __attribute__((ext_vector_type(4))) short ra_s16x4_t;
+typedef __attribute__((address_space(3))) ra_s16x4_t ra_lds_s16x4_t;
 #define RM_KT 32
 
 __device__ __forceinline__ ra_bf16x8_t ra_load8(const bf16_t* p) { return *reinterpret_cast<const ra_bf16x8_t*>(p); }
@@ -336,17 +338,22 @@ __device__ __forceinline__ int ra_oldest_seen(int kind, int size, int pos) {
   return 0;
 }
 
-template <int D32, int NT, int UPW, int MAPS>
+// ALIAS: the values are columns of the key tile (one plane, one map): no value tile, no value loads.
+template <int D32, int NT, int UPW, int MAPS, bool ALIAS>
 __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, const RowsMfmaExtra x) {
   extern __shared__ __align__(16) unsigned char ra_smem[];
   constexpr int D = D32 * 32, DA = D * MAPS, VW = NT * 16;
-  constexpr int KROW = DA + 8, VROW = RM_KT + 8;
+  // rows of both tiles are padded so that the 16-byte reads of key fragments and the 8-byte
+  // transposing reads of value fragments spread over the banks
+  constexpr int KROW = DA + 8, VROW = VW + 16;
   constexpr int KPR = DA / 8, VPR = VW / 8;
-  constexpr int PFK = (RM_KT * KPR + 255) / 256, PFV = (RM_KT * VPR + 255) / 256;
+  constexpr int PFK = (RM_KT * KPR + 255) / 256, PFV = ALIAS ? 1 : (RM_KT * VPR + 255) / 256;
   static_assert(MAPS == 1 || UPW == 2, "two maps: a wave holds the two maps of one head");
+  static_assert(!ALIAS || MAPS == 1, "values inside the key row: one map");
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int l16 = lane & 15, slot = lane >> 4;
-  const int* item = p.items + 4 * (int64_t)blockIdx.x;
+  // items come with a request's tokens in order; the last ones see the most keys and go first
+  const int* item = p.items + 4 * (int64_t)(gridDim.x - 1 - blockIdx.x);
   const int req = item[0], tok0 = item[1];
   const int q_len = p.cu_q[req + 1] - p.cu_q[req];
   if (tok0 >= q_len) return;  // an item past the request's tokens (a batch of fixed shape)
@@ -365,10 +372,9 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
   const int h0 = hc * x.heads_per_wg;
   const int nh_here = min(x.heads_per_wg, group - h0);
   const int v0 = vs * VW;
-  const bool alias = p.v_plane == p.k_plane;
 
   bf16_t* Ks = reinterpret_cast<bf16_t*>(ra_smem);   // [RM_KT][KROW]
-  bf16_t* Vt = Ks + RM_KT * KROW;                    // [VW][VROW]
+  bf16_t* Vs = Ks + RM_KT * KROW;                    // [RM_KT][VROW], row-major (not with ALIAS)
   const bf16_t* q = (const bf16_t*)p.q;
   const bf16_t* kc = (const bf16_t*)p.k_plane;
   const bf16_t* vc = (const bf16_t*)p.v_plane;
@@ -413,38 +419,29 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
       const uint4 v = *reinterpret_cast<const uint4*>(kc + (row >= 0 ? row : 0) * p.k_row + (int64_t)g * DA + e * 8);
       kreg[it] = (row >= 0 && idx == at) ? v : make_uint4(0, 0, 0, 0);
     }
+    if constexpr (!ALIAS) {
 #pragma unroll
-    for (int it = 0; it < PFV; ++it) {
-      const int idx = tid + it * 256;
-      const int at = min(idx, RM_KT * VPR - 1);
-      const int e = at % VPR, jj = at / VPR;
-      const int64_t row = row_of(k0 + jj);
-      const int64_t col = alias ? (int64_t)v0 : (int64_t)g * p.vdim + v0;
-      const uint4 v = *reinterpret_cast<const uint4*>(vc + (row >= 0 ? row : 0) * p.v_row + col + e * 8);
-      vreg[it] = (row >= 0 && idx == at) ? v : make_uint4(0, 0, 0, 0);
+      for (int it = 0; it < PFV; ++it) {
+        const int idx = tid + it * 256;
+        const int at = min(idx, RM_KT * VPR - 1);
+        const int e = at % VPR, jj = at / VPR;
+        const int64_t row = row_of(k0 + jj);
+        const uint4 v = *reinterpret_cast<const uint4*>(vc + (row >= 0 ? row : 0) * p.v_row + (int64_t)g * p.vdim + v0 + e * 8);
+        vreg[it] = (row >= 0 && idx == at) ? v : make_uint4(0, 0, 0, 0);
+      }
     }
   };
   auto store = [&]() {
 #pragma unroll
     for (int it = 0; it < PFK; ++it) {
       const int idx = tid + it * 256;
-      if (idx < RM_KT * KPR) {
-        const int e = idx % KPR, jj = idx / KPR;
-        *reinterpret_cast<uint4*>(Ks + jj * KROW + e * 8) = kreg[it];
-      }
+      if (idx < RM_KT * KPR) *reinterpret_cast<uint4*>(Ks + (idx / KPR) * KROW + (idx % KPR) * 8) = kreg[it];
     }
+    if constexpr (!ALIAS) {
 #pragma unroll
-    for (int it = 0; it < PFV; ++it) {
-      const int idx = tid + it * 256;
-      if (idx < RM_KT * VPR) {
-        const int e = idx % VPR, jj = idx / VPR;
-        const uint32_t w[4] = {vreg[it].x, vreg[it].y, vreg[it].z, vreg[it].w};
-        uint16_t* dst = reinterpret_cast<uint16_t*>(Vt) + (e * 8) * VROW + jj;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          dst[(2 * u) * VROW] = (uint16_t)(w[u] & 0xffffu);
-          dst[(2 * u + 1) * VROW] = (uint16_t)(w[u] >> 16);
-        }
+      for (int it = 0; it < PFV; ++it) {
+        const int idx = tid + it * 256;
+        if (idx < RM_KT * VPR) *reinterpret_cast<uint4*>(Vs + (idx / VPR) * VROW + (idx % VPR) * 8) = vreg[it];
       }
     }
   };
@@ -462,6 +459,13 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) out[a][nt] = ra_f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
   }
+  // where this lane's value fragments begin: the transposing read (ds_read_b64_tr_b16) hands lane i
+  // of a group of 16 element i % 4 of what lanes i / 4, 4 + i / 4, 8 + i / 4 and 12 + i / 4 address; with
+  // lane i pointing at key 4 * slot + i / 4, columns 4 * (i % 4) .. + 4 of a 16-wide block, every lane
+  // receives its column (i) of the keys 4 * slot .. + 4: the order in which it holds its weights
+  const bf16_t* vlane = ALIAS ? Ks + (4 * slot + (l16 >> 2)) * KROW + v0 + 4 * (l16 & 3)
+                              : Vs + (4 * slot + (l16 >> 2)) * VROW + 4 * (l16 & 3);
+  constexpr int VSTRIDE = ALIAS ? KROW : VROW;
 
   if (c_begin < c_end) fetch(first + c_begin * RM_KT);
   for (int c = c_begin; c < c_end; ++c) {
@@ -520,10 +524,10 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
     // values: a fragment (16 value columns, 32 keys) serves all of the wave's units
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const bf16_t* vb = Vt + (nt * 16 + l16) * VROW + slot * 4;
-      const uint2 lo4 = *reinterpret_cast<const uint2*>(vb), hi4 = *reinterpret_cast<const uint2*>(vb + 16);
-      const uint4 both = make_uint4(lo4.x, lo4.y, hi4.x, hi4.y);
-      const ra_bf16x8_t vf = *reinterpret_cast<const ra_bf16x8_t*>(&both);
+      const bf16_t* vp = vlane + nt * 16;
+      const ra_s16x4_t f0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ra_lds_s16x4_t*)vp);
+      const ra_s16x4_t f1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ra_lds_s16x4_t*)(vp + 16 * VSTRIDE));
+      const ra_bf16x8_t vf = __builtin_bit_cast(ra_bf16x8_t, __builtin_shufflevector(f0, f1, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
       for (int a = 0; a < UPW; ++a) out[a][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pw[a], vf, out[a][nt], 0, 0, 0);
     }
@@ -531,7 +535,7 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
 
   if (runs > 1) {
     // maximum, denominator and unnormalised sums of this run, per unit and query
-    const int64_t wg = ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * runs + blockIdx.z;
+    const int64_t wg = ((int64_t)(gridDim.x - 1 - blockIdx.x) * gridDim.y + blockIdx.y) * runs + blockIdx.z;
     float* base = x.workspace + wg * (4 * UPW * 16 * (2 + VW));
 #pragma unroll
     for (int a = 0; a < UPW; ++a) {
@@ -593,12 +597,14 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
   }
 }
 
-// Puts the runs of rows_mfma_kernel together: one workgroup per (item, key/value head, head chunk,
-// value split); a thread takes one query (tid / 16) and the value columns tid % 16 + 16 i.
+// Puts the runs of rows_mfma_kernel together: one workgroup per (item, key/value head x head chunk x
+// value split, head of the chunk); per query of the item a thread takes the value columns tid,
+// tid + 256.
 template <int MAPS>
 __global__ __launch_bounds__(256) void rows_merge_kernel(const RowsAttnParams p, const RowsMfmaExtra x, int runs, int upw,
                                                          int vw) {
-  const int tid = threadIdx.x, qi = tid >> 4, sub = tid & 15;
+  __shared__ float scratch[4];
+  const int tid = threadIdx.x;
   const int* item = p.items + 4 * (int64_t)blockIdx.x;
   const int req = item[0], tok0 = item[1];
   const int q_len = p.cu_q[req + 1] - p.cu_q[req];
@@ -610,94 +616,91 @@ __global__ __launch_bounds__(256) void rows_merge_kernel(const RowsAttnParams p,
   const int g = blockIdx.y / (x.v_splits * x.head_chunks);
   const int group = p.heads / p.kv_heads;
   const int h0 = hc * x.heads_per_wg;
-  const int nh_here = min(x.heads_per_wg, group - h0);
+  const int hl = blockIdx.z;
+  if (hl >= min(x.heads_per_wg, group - h0)) return;
+  const int head = g * group + h0 + hl;
   const int v0 = vs * vw;
-  const int stride_q = 2 + vw, stride_unit = 16 * stride_q, stride_run = 4 * upw * stride_unit;
+  const int stride_q = 2 + vw, stride_unit = 16 * stride_q;
+  const int64_t stride_run = (int64_t)4 * upw * stride_unit;
   const float* base = x.workspace + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * runs * stride_run;
   const float lam = (MAPS == 2 && p.lambda) ? p.lambda[0] : 0.0f;
   bf16_t* o = (bf16_t*)p.out;
-  for (int hl = 0; hl < nh_here; ++hl) {
-    float val[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) val[i] = 0.0f;
+  for (int qi = 0; qi < nq; ++qi) {
+    float val[2] = {0.0f, 0.0f};
 #pragma unroll
     for (int map = 0; map < MAPS; ++map) {
       // the unit's place in a run's block: (wave, a)
       const int unit = MAPS == 2 ? hl * upw + map : (hl % 4) * upw + hl / 4;
       const float* u = base + (int64_t)unit * stride_unit + qi * stride_q;
       float top = -3.0e38f;
-      for (int r = 0; r < runs; ++r) top = fmaxf(top, u[(int64_t)r * stride_run]);
-      float den = 0.0f;
-      float part[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) part[i] = 0.0f;
+      for (int r = 0; r < runs; ++r) top = fmaxf(top, u[r * stride_run]);
+      float den = 0.0f, part[2] = {0.0f, 0.0f};
       for (int r = 0; r < runs; ++r) {
-        const float* ur = u + (int64_t)r * stride_run;
+        const float* ur = u + r * stride_run;
         const float f = __builtin_amdgcn_exp2f(ur[0] - top);
         den += ur[1] * f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
-          if (sub + 16 * i < vw) part[i] += ur[2 + sub + 16 * i] * f;
+        for (int i = 0; i < 2; ++i)
+          if (tid + 256 * i < vw) part[i] += ur[2 + tid + 256 * i] * f;
       }
       const float inv = den > 0.0f ? 1.0f / den : 0.0f;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) val[i] += (map == 0 ? 1.0f : -lam) * part[i] * inv;
+      for (int i = 0; i < 2; ++i) val[i] += (map == 0 ? 1.0f : -lam) * part[i] * inv;
     }
     float mult = 1.0f;
     if (p.head_norm) {
-      float sq = 0.0f;
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (sub + 16 * i < vw) sq += val[i] * val[i];
-#pragma unroll
-      for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+      float sq = cw_wave_sum(val[0] * val[0] + val[1] * val[1]);   // columns past vw hold zeros
+      __syncthreads();
+      if ((tid & 63) == 0) scratch[tid >> 6] = sq;
+      __syncthreads();
+      sq = (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
       mult = p.post_mult / sqrtf(sq / (float)p.vdim + p.norm_eps);
     }
-    if (qi < nq) {
-      const int head = g * group + h0 + hl;
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (sub + 16 * i < vw)
-          o[(row0 + qi) * p.out_stride + (int64_t)head * p.out_head_stride + v0 + sub + 16 * i] = __float2bfloat16(val[i] * mult);
-    }
+    for (int i = 0; i < 2; ++i)
+      if (tid + 256 * i < vw)
+        o[(row0 + qi) * p.out_stride + (int64_t)head * p.out_head_stride + v0 + tid + 256 * i] = __float2bfloat16(val[i] * mult);
   }
 }
 
 // How the matrix-core kernel cuts a geometry: value columns a workgroup takes (16 * nt), how many
-// workgroups share the columns, units a wave holds; 0 in *nt: not taken. Key rows of 32 * d32
-// elements a map for d32 in {2, 4} (two maps) or {5, 10, 18} (one map), value rows of 64, 128 or 256
-// (two maps: the head norm needs all columns in one workgroup) or 128, 256, 512 (one map).
-static void ra_mfma_shape(int maps, int dim, int vdim, int* d32, int* nt, int* v_splits, int* upw) {
+// workgroups share the columns, units a wave holds; 0 in *nt: not taken. Two maps: key rows of 64
+// or 128 elements a map, value rows of 64, 128 or 256 (the head norm needs all columns in one
+// workgroup). One map with the values inside the key row: key rows of 160, 320 or 576 elements,
+// values their first 128, 256 or 512.
+static void ra_mfma_shape(int maps, int dim, int vdim, int alias, int* d32, int* nt, int* v_splits, int* upw) {
   *nt = 0; *v_splits = 1; *upw = maps == 2 ? 2 : 1; *d32 = dim / 32;
   if (dim % 32) return;
-  if (maps == 2) {
+  if (maps == 2 && !alias) {
     if (*d32 != 2 && *d32 != 4) return;
     if (vdim == 64) *nt = 4; else if (vdim == 128) *nt = 8; else if (vdim == 256) *nt = 16;
-  } else {
-    if (*d32 != 5 && *d32 != 10 && *d32 != 18) return;
-    if (vdim == 128) *nt = 8; else if (vdim == 256) *nt = 16; else if (vdim == 512) { *nt = 16; *v_splits = 2; }
+  } else if (maps == 1 && alias) {
+    if (*d32 == 5 && vdim == 128) *nt = 8;
+    else if (*d32 == 10 && vdim == 256) *nt = 16;
+    else if (*d32 == 18 && vdim == 512) *nt = 32;
   }
 }
 
-CW_EXPORT int cw_rows_mfma_supported(int maps, int dim, int vdim) {
+CW_EXPORT int cw_rows_mfma_supported(int maps, int dim, int vdim, int alias) {
   int d32, nt, vsp, upw;
-  ra_mfma_shape(maps, dim, vdim, &d32, &nt, &vsp, &upw);
+  ra_mfma_shape(maps, dim, vdim, alias, &d32, &nt, &vsp, &upw);
   return nt != 0;
 }
 
 // Workgroups of one run of keys: (items, y); and the floats of workspace that ``runs`` runs need.
-CW_EXPORT int cw_rows_mfma_grid_y(int heads, int kv_heads, int maps, int dim, int vdim) {
+CW_EXPORT int cw_rows_mfma_grid_y(int heads, int kv_heads, int maps, int dim, int vdim, int alias) {
   int d32, nt, vsp, upw;
-  ra_mfma_shape(maps, dim, vdim, &d32, &nt, &vsp, &upw);
+  ra_mfma_shape(maps, dim, vdim, alias, &d32, &nt, &vsp, &upw);
   if (!nt || heads % kv_heads) return 0;
   const int per_wg = maps == 2 ? 4 : 4 * upw, group = heads / kv_heads;
   return kv_heads * ((group + per_wg - 1) / per_wg) * vsp;
 }
-CW_EXPORT int64_t cw_rows_mfma_workspace_floats(int n_items, int heads, int kv_heads, int maps, int dim, int vdim, int runs) {
+CW_EXPORT int64_t cw_rows_mfma_workspace_floats(int n_items, int heads, int kv_heads, int maps, int dim, int vdim, int alias,
+                                                int runs) {
   int d32, nt, vsp, upw;
-  ra_mfma_shape(maps, dim, vdim, &d32, &nt, &vsp, &upw);
+  ra_mfma_shape(maps, dim, vdim, alias, &d32, &nt, &vsp, &upw);
   if (!nt || runs <= 1) return 0;
-  return (int64_t)n_items * cw_rows_mfma_grid_y(heads, kv_heads, maps, dim, vdim) * runs * 4 * upw * 16 * (2 + 16 * nt);
+  return (int64_t)n_items * cw_rows_mfma_grid_y(heads, kv_heads, maps, dim, vdim, alias) * runs * 4 * upw * 16 * (2 + 16 * nt);
 }
 
 CW_EXPORT int cw_rows_attention_mfma(const void* q, int64_t q_stride, int64_t q_head_stride, void* out, int64_t out_stride,
@@ -710,17 +713,17 @@ CW_EXPORT int cw_rows_attention_mfma(const void* q, int64_t q_stride, int64_t q_
   if (n_items < 0 || !q || !out || !k_plane || !v_plane || !block_tables || !ctx_lens || !cu_q || !items) return CW_ERR_ARG;
   if (block_size <= 0 || table_width <= 0 || mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && mask_size < 1)) return CW_ERR_ARG;
   if ((maps == 2 && !lambda) || runs < 1 || runs > 64) return CW_ERR_ARG;
-  int d32, nt, vsp, upw;
-  ra_mfma_shape(maps, dim, vdim, &d32, &nt, &vsp, &upw);
-  if (!nt || heads % kv_heads) return CW_ERR_SIZE;
   const int alias = v_plane == k_plane;
+  int d32, nt, vsp, upw;
+  ra_mfma_shape(maps, dim, vdim, alias, &d32, &nt, &vsp, &upw);
+  if (!nt || heads % kv_heads) return CW_ERR_SIZE;
   if (alias && (maps != 1 || kv_heads != 1 || vdim > dim)) return CW_ERR_ARG;
   if (head_norm && vsp != 1) return CW_ERR_ARG;
   // 16-byte loads: rows and heads begin at multiples of 8 elements
   if (q_stride % 8 || q_head_stride % 8 || k_row % 8 || (!alias && v_row % 8) || ((uintptr_t)q | (uintptr_t)k_plane | (uintptr_t)v_plane) % 16)
     return CW_ERR_ARG;
   if (k_row < kv_heads * maps * dim || (!alias && v_row < kv_heads * vdim)) return CW_ERR_ARG;
-  if (runs > 1 && (!workspace || workspace_floats < cw_rows_mfma_workspace_floats(n_items, heads, kv_heads, maps, dim, vdim, runs)))
+  if (runs > 1 && (!workspace || workspace_floats < cw_rows_mfma_workspace_floats(n_items, heads, kv_heads, maps, dim, vdim, alias, runs)))
     return CW_ERR_ARG;
   if (n_items == 0) return CW_OK;
   RowsAttnParams p;
@@ -736,33 +739,30 @@ CW_EXPORT int cw_rows_attention_mfma(const void* q, int64_t q_stride, int64_t q_
   const int group = heads / kv_heads;
   x.head_chunks = (group + x.heads_per_wg - 1) / x.heads_per_wg;
   dim3 grid(n_items, kv_heads * x.head_chunks * vsp, runs), block(256);
-  const size_t smem = ((size_t)RM_KT * (maps * dim + 8) + (size_t)16 * nt * (RM_KT + 8)) * 2;
-#define CW_LAUNCH(D32_, NT_, UPW_, MAPS_)                                                                          \
+  const size_t smem = ((size_t)RM_KT * (maps * dim + 8) + (alias ? 0 : (size_t)RM_KT * (16 * nt + 16))) * 2;
+#define CW_LAUNCH(D32_, NT_, UPW_, MAPS_, ALIAS_)                                                                  \
   do {                                                                                                             \
-    if (smem > 48 * 1024 && hipFuncSetAttribute((const void*)rows_mfma_kernel<D32_, NT_, UPW_, MAPS_>,             \
+    if (smem > 48 * 1024 && hipFuncSetAttribute((const void*)rows_mfma_kernel<D32_, NT_, UPW_, MAPS_, ALIAS_>,     \
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) \
       return CW_ERR_LAUNCH;                                                                                        \
-    hipLaunchKernelGGL((rows_mfma_kernel<D32_, NT_, UPW_, MAPS_>), grid, block, smem, stream, p, x);               \
-  } while (0)
-#define CW_PICK_NT(D32_, UPW_, MAPS_, A_, B_, C_)                                                                  \
-  do {                                                                                                             \
-    if (nt == A_) CW_LAUNCH(D32_, A_, UPW_, MAPS_);                                                                \
-    else if (nt == B_) CW_LAUNCH(D32_, B_, UPW_, MAPS_);                                                           \
-    else CW_LAUNCH(D32_, C_, UPW_, MAPS_);                                                                         \
+    hipLaunchKernelGGL((rows_mfma_kernel<D32_, NT_, UPW_, MAPS_, ALIAS_>), grid, block, smem, stream, p, x);       \
   } while (0)
   if (maps == 2) {
-    if (d32 == 2) CW_PICK_NT(2, 2, 2, 4, 8, 16);
-    else CW_PICK_NT(4, 2, 2, 4, 8, 16);
+    if (d32 == 2 && nt == 4) CW_LAUNCH(2, 4, 2, 2, false);
+    else if (d32 == 2 && nt == 8) CW_LAUNCH(2, 8, 2, 2, false);
+    else if (d32 == 2) CW_LAUNCH(2, 16, 2, 2, false);
+    else if (nt == 4) CW_LAUNCH(4, 4, 2, 2, false);
+    else if (nt == 8) CW_LAUNCH(4, 8, 2, 2, false);
+    else CW_LAUNCH(4, 16, 2, 2, false);
   } else {
-    if (d32 == 5) CW_PICK_NT(5, 1, 1, 8, 16, 16);
-    else if (d32 == 10) CW_PICK_NT(10, 1, 1, 8, 16, 16);
-    else CW_PICK_NT(18, 1, 1, 8, 16, 16);
+    if (d32 == 5) CW_LAUNCH(5, 8, 1, 1, true);
+    else if (d32 == 10) CW_LAUNCH(10, 16, 1, 1, true);
+    else CW_LAUNCH(18, 32, 1, 1, true);
   }
-#undef CW_PICK_NT
 #undef CW_LAUNCH
   if (hipGetLastError() != hipSuccess) return CW_ERR_LAUNCH;
   if (runs > 1) {
-    dim3 mgrid(n_items, grid.y);
+    dim3 mgrid(n_items, grid.y, x.heads_per_wg);
     if (maps == 2) hipLaunchKernelGGL(rows_merge_kernel<2>, mgrid, block, 0, stream, p, x, runs, upw, 16 * nt);
     else hipLaunchKernelGGL(rows_merge_kernel<1>, mgrid, block, 0, stream, p, x, runs, upw, 16 * nt);
   }

@@ -137,9 +137,9 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_rows_attention_key_chunk": [I, I, I, I],
             "cw_rows_attention_heads_per_group": [I, I, I],
             "cw_rows_attention_tokens_per_item": [I, I, I],
-            "cw_rows_mfma_supported": [I, I, I],
-            "cw_rows_mfma_grid_y": [I, I, I, I, I],
-            "cw_rows_mfma_workspace_floats": [I, I, I, I, I, I, I],
+            "cw_rows_mfma_supported": [I, I, I, I],
+            "cw_rows_mfma_grid_y": [I, I, I, I, I, I],
+            "cw_rows_mfma_workspace_floats": [I, I, I, I, I, I, I, I],
             "cw_rows_attention_mfma": [P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F,
                                        I, P, L, P],
             "cw_rows_attention": [I, P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F, P],
@@ -1693,19 +1693,19 @@ def rows_attention_tokens_per_item(heads: int, kv_heads: int, maps: int = 1) -> 
 ROWS_MFMA_TOKENS = 16   # tokens of one request that a work item of the matrix-core kernel holds
 
 
-def rows_mfma_supported(dim: int, vdim: int, maps: int, dtype) -> bool:
-    """Does the matrix-core kernel take this geometry? bfloat16; key rows of 64 or 128 elements a
-    map with value rows of 64, 128 or 256 (two maps), key rows of 160, 320 or 576 with value rows
-    of 128, 256 or 512 (one map)."""
-    return dtype == torch.bfloat16 and bool(_load("rows_attention").cw_rows_mfma_supported(maps, dim, vdim))
+def rows_mfma_supported(dim: int, vdim: int, maps: int, dtype, alias: bool = False) -> bool:
+    """Does the matrix-core kernel take this geometry? bfloat16; two maps with key rows of 64 or
+    128 elements a map and value rows of 64, 128 or 256; or one map whose values lie inside the
+    key row (``alias``): key rows of 160, 320 or 576 elements, values their first 128, 256 or 512."""
+    return dtype == torch.bfloat16 and bool(_load("rows_attention").cw_rows_mfma_supported(maps, dim, vdim, int(alias)))
 
 
 def rows_mfma_key_runs(n_items: int, longest: int, heads: int, kv_heads: int, dim: int, vdim: int, maps: int,
-                       compute_units: int) -> int:
+                       compute_units: int, alias: bool = False) -> int:
     """Into how many runs the matrix-core kernel cuts every item's keys: as many as there are idle
     compute units for while the longest key range gives each run 128 keys, 64 at most (a step of
     single tokens, or a short portion behind a long context, would leave most of the card idle)."""
-    per_run = n_items * int(_load("rows_attention").cw_rows_mfma_grid_y(heads, kv_heads, maps, dim, vdim))
+    per_run = n_items * int(_load("rows_attention").cw_rows_mfma_grid_y(heads, kv_heads, maps, dim, vdim, int(alias)))
     if per_run <= 0:
         return 1
     return int(max(1, min(compute_units // per_run, longest // 128, 64)))
@@ -1788,8 +1788,8 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
     _need(mask in MASK_KINDS and (mask == "causal" or mask_size >= 1), f"mask {mask!r} of size {mask_size}")
     if mfma:
         lib = _load("rows_attention")
-        _need(rows_mfma_supported(dim, vdim, maps, q.dtype), "the matrix-core kernel does not take this geometry")
-        need = int(lib.cw_rows_mfma_workspace_floats(n_items, heads, kv_heads, maps, dim, vdim, key_runs))
+        _need(rows_mfma_supported(dim, vdim, maps, q.dtype, alias), "the matrix-core kernel does not take this geometry")
+        need = int(lib.cw_rows_mfma_workspace_floats(n_items, heads, kv_heads, maps, dim, vdim, int(alias), key_runs))
         workspace = torch.empty(need, dtype=torch.float32, device=q.device) if need else None
         _check(lib.cw_rows_attention_mfma(
             _ptr(q), qs, qh, _ptr(out), os_, oh, _ptr(k_plane), _ptr(k_plane if alias else v_plane), k2.shape[1], v_row, rows,

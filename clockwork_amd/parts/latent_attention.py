@@ -75,7 +75,7 @@ class LatentAttention(Part):
             raise ValueError(f"latent attention with rows of {self.row} elements is beyond the attention kernel for paged rows "
                              "(a latent of up to 512 elements, tiles of 150 KB of LDS)")
         # bfloat16 with the common latent sizes runs on the matrix cores
-        self.mfma = ops.rows_mfma_supported(self.row, s.kv_rank, 1, dtype)
+        self.mfma = ops.rows_mfma_supported(self.row, s.kv_rank, 1, dtype, alias=True)
         self.run = ops.ROWS_MFMA_TOKENS if self.mfma else ops.rows_attention_tokens_per_item(s.num_heads, 1, 1)
 
     def _plan(self, ctx):
@@ -88,7 +88,7 @@ class LatentAttention(Part):
             runs = 1
             if self.mfma:
                 runs = ops.rows_mfma_key_runs(n_items, longest_key_range(ctx, s.window), s.num_heads, 1, self.row, s.kv_rank, 1,
-                                              ctx.num_compute_units)
+                                              ctx.num_compute_units, alias=True)
             plan = ctx.plans[key] = (items, n_items, runs)
         return plan
 

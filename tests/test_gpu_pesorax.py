@@ -259,9 +259,10 @@ def _latent_sizes(spec):
 
 
 # heads, dim, rot_dim, rot dims, vdim, q_rank, kv_rank, hidden: partial rotation, sizes of 1 and 2, more
-# heads than a workgroup takes at once, a latent of 256 + 64 elements
+# heads than a workgroup takes at once, latents of 256 + 64 and 512 + 64 elements
 LATENT_SHAPES = [(3, 24, 16, 8, 20, 40, 48, 96), (1, 2, 2, 2, 1, 4, 8, 48), (5, 8, 4, 4, 12, 20, 36, 100),
-                 (20, 8, 8, 8, 8, 16, 16, 64), (4, 32, 64, 64, 32, 48, 256, 64), (2, 16, 8, 0, 16, 12, 24, 64)]
+                 (20, 8, 8, 8, 8, 16, 16, 64), (4, 32, 64, 64, 32, 48, 256, 64), (2, 16, 8, 0, 16, 12, 24, 64),
+                 (5, 16, 64, 64, 16, 32, 512, 64)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
