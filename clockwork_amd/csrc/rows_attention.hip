@@ -402,21 +402,25 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
   const int c_begin = blockIdx.z * per_run, c_end = min(n_chunks, c_begin + per_run);
 
   uint4 kreg[PFK], vreg[PFV];
-  auto row_of = [&](int j) -> int64_t {
+  // A chunk's cache rows are looked up once, by 32 threads, and wait in LDS (two chunks' worth):
+  // a lookup inside the fetch would put a load of the page table before every load of a row, and
+  // since loads come home in order each row's load would wait for all the loads before it.
+  __shared__ int chunk_rows[2][RM_KT];
+  auto row_of = [&](int j) -> int {
     if (j > last) return -1;
     const int b = j / p.block_size;
     const int page = b < p.table_width ? table[b] : -1;
     const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
-    return (page >= 0 && row < p.cache_rows) ? row : -1;
+    return (page >= 0 && row < p.cache_rows) ? (int)row : -1;
   };
-  auto fetch = [&](int k0) {
+  auto fetch = [&](const int* rows_of_chunk) {
 #pragma unroll
     for (int it = 0; it < PFK; ++it) {
       const int idx = tid + it * 256;
       const int at = min(idx, RM_KT * KPR - 1);
       const int e = at % KPR, jj = at / KPR;
-      const int64_t row = row_of(k0 + jj);
-      const uint4 v = *reinterpret_cast<const uint4*>(kc + (row >= 0 ? row : 0) * p.k_row + (int64_t)g * DA + e * 8);
+      const int row = rows_of_chunk[jj];
+      const uint4 v = *reinterpret_cast<const uint4*>(kc + (int64_t)(row >= 0 ? row : 0) * p.k_row + (int64_t)g * DA + e * 8);
       kreg[it] = (row >= 0 && idx == at) ? v : make_uint4(0, 0, 0, 0);
     }
     if constexpr (!ALIAS) {
@@ -425,8 +429,8 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
         const int idx = tid + it * 256;
         const int at = min(idx, RM_KT * VPR - 1);
         const int e = at % VPR, jj = at / VPR;
-        const int64_t row = row_of(k0 + jj);
-        const uint4 v = *reinterpret_cast<const uint4*>(vc + (row >= 0 ? row : 0) * p.v_row + (int64_t)g * p.vdim + v0 + e * 8);
+        const int row = rows_of_chunk[jj];
+        const uint4 v = *reinterpret_cast<const uint4*>(vc + (int64_t)(row >= 0 ? row : 0) * p.v_row + (int64_t)g * p.vdim + v0 + e * 8);
         vreg[it] = (row >= 0 && idx == at) ? v : make_uint4(0, 0, 0, 0);
       }
     }
@@ -467,13 +471,22 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
                               : Vs + (4 * slot + (l16 >> 2)) * VROW + 4 * (l16 & 3);
   constexpr int VSTRIDE = ALIAS ? KROW : VROW;
 
-  if (c_begin < c_end) fetch(first + c_begin * RM_KT);
+  if (c_begin < c_end) {
+    if (tid < RM_KT) chunk_rows[0][tid] = row_of(first + c_begin * RM_KT + tid);
+    if (tid >= 64 && tid < 64 + RM_KT && c_begin + 1 < c_end) chunk_rows[1][tid - 64] = row_of(first + (c_begin + 1) * RM_KT + tid - 64);
+    __syncthreads();
+    fetch(chunk_rows[0]);
+  }
   for (int c = c_begin; c < c_end; ++c) {
     const int k0 = first + c * RM_KT;
-    __syncthreads();
+    __syncthreads();   // the tiles of the chunk before have been read; the rows of the next chunk are written
     store();
-    if (c + 1 < c_end) fetch(k0 + RM_KT);
+    if (c + 1 < c_end) fetch(chunk_rows[(c + 1 - c_begin) & 1]);
     __syncthreads();
+    // the rows of the chunk after the next: looked up now, written at the end of this round
+    int later_row = -1;
+    const bool looks_up = tid < RM_KT && c + 2 < c_end;
+    if (looks_up) later_row = row_of(k0 + 2 * RM_KT + tid);
     const bool inside = nq == 16 && k0 + RM_KT - 1 <= pos0 && k0 >= lo_last;
     ra_bf16x8_t pw[UPW];
 #pragma unroll
@@ -531,6 +544,7 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
 #pragma unroll
       for (int a = 0; a < UPW; ++a) out[a][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pw[a], vf, out[a][nt], 0, 0, 0);
     }
+    if (looks_up) chunk_rows[(c - c_begin) & 1][tid] = later_row;   // this chunk's rows were last read before this round's second barrier
   }
 
   if (runs > 1) {
@@ -625,20 +639,32 @@ __global__ __launch_bounds__(256) void rows_merge_kernel(const RowsAttnParams p,
   const float* base = x.workspace + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * runs * stride_run;
   const float lam = (MAPS == 2 && p.lambda) ? p.lambda[0] : 0.0f;
   bf16_t* o = (bf16_t*)p.out;
+  __shared__ float run_stats[2][64][2];   // per map and run: maximum (in units of log 2) and denominator
   for (int qi = 0; qi < nq; ++qi) {
     float val[2] = {0.0f, 0.0f};
+    // every run's maximum and denominator, fetched side by side
+    __syncthreads();
+    if (tid < MAPS * runs) {
+      const int map = tid / runs, r = tid % runs;
+      const int unit = MAPS == 2 ? hl * upw + map : (hl % 4) * upw + hl / 4;
+      const float* u = base + (int64_t)unit * stride_unit + qi * stride_q + r * stride_run;
+      run_stats[map][r][0] = u[0];
+      run_stats[map][r][1] = u[1];
+    }
+    __syncthreads();
 #pragma unroll
     for (int map = 0; map < MAPS; ++map) {
       // the unit's place in a run's block: (wave, a)
       const int unit = MAPS == 2 ? hl * upw + map : (hl % 4) * upw + hl / 4;
       const float* u = base + (int64_t)unit * stride_unit + qi * stride_q;
       float top = -3.0e38f;
-      for (int r = 0; r < runs; ++r) top = fmaxf(top, u[r * stride_run]);
+      for (int r = 0; r < runs; ++r) top = fmaxf(top, run_stats[map][r][0]);
       float den = 0.0f, part[2] = {0.0f, 0.0f};
+#pragma unroll 4
       for (int r = 0; r < runs; ++r) {
         const float* ur = u + r * stride_run;
-        const float f = __builtin_amdgcn_exp2f(ur[0] - top);
-        den += ur[1] * f;
+        const float f = __builtin_amdgcn_exp2f(run_stats[map][r][0] - top);
+        den += run_stats[map][r][1] * f;
 #pragma unroll
         for (int i = 0; i < 2; ++i)
           if (tid + 256 * i < vw) part[i] += ur[2 + tid + 256 * i] * f;
