@@ -360,6 +360,43 @@ __global__ __launch_bounds__(256) void add_dyt_kernel(float* __restrict__ resid,
   }
 }
 
+// The same for bfloat16 rows of a multiple of 4 elements: a thread takes 4 neighbours (16 bytes of
+// the stream, 8 of the branch and of the output).
+template <typename WT>
+__global__ __launch_bounds__(256) void add_dyt_vec4_kernel(float* __restrict__ resid, const bf16_t* __restrict__ delta,
+                                                           float scale, const float* __restrict__ extra,
+                                                           const WT* __restrict__ w, const WT* __restrict__ b,
+                                                           const float* __restrict__ alpha, bf16_t* __restrict__ out,
+                                                           const int* __restrict__ rows, int H) {
+  const int64_t i = blockIdx.x;
+  const int64_t src = rows ? (int64_t)rows[i] : i;
+  const float a = alpha[0];
+  for (int j = 4 * threadIdx.x; j < H; j += 4 * 256) {
+    float4 x = *reinterpret_cast<const float4*>(resid + src * H + j);
+    if (delta) {
+      const uint2 d = *reinterpret_cast<const uint2*>(delta + src * H + j);
+      x.x += scale * cw_bf16_bits_to_float((uint16_t)(d.x & 0xffffu));
+      x.y += scale * cw_bf16_bits_to_float((uint16_t)(d.x >> 16));
+      x.z += scale * cw_bf16_bits_to_float((uint16_t)(d.y & 0xffffu));
+      x.w += scale * cw_bf16_bits_to_float((uint16_t)(d.y >> 16));
+    }
+    if (extra) {
+      const float4 e = *reinterpret_cast<const float4*>(extra + src * H + j);
+      x.x += e.x; x.y += e.y; x.z += e.z; x.w += e.w;
+    }
+    if (!rows && (delta || extra)) *reinterpret_cast<float4*>(resid + src * H + j) = x;
+    const float xs[4] = {x.x, x.y, x.z, x.w};
+    uint16_t y[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float v = tanhf(a * xs[u]) * cw_to_float(w[j + u]);
+      if (b) v += cw_to_float(b[j + u]);
+      y[u] = cw_float_to_bf16_bits(v);
+    }
+    *reinterpret_cast<uint2*>(out + i * H + j) = make_uint2((uint32_t)y[0] | ((uint32_t)y[1] << 16), (uint32_t)y[2] | ((uint32_t)y[3] << 16));
+  }
+}
+
 CW_EXPORT int cw_add_dyt(float* resid, const void* delta, int delta_dtype, float scale, const float* extra, const void* w,
                          const void* b, int w_dtype, const float* alpha, void* out, int out_dtype, const int* rows, int n,
                          int H, hipStream_t stream) {
@@ -370,7 +407,15 @@ CW_EXPORT int cw_add_dyt(float* resid, const void* delta, int delta_dtype, float
   hipLaunchKernelGGL((add_dyt_kernel<DT_, WT_, OT_>), grid, block, 0, stream, resid, (const DT_*)delta, scale, extra, \
                      (const WT_*)w, (const WT_*)b, alpha, (OT_*)out, rows, H)
   const int dd = delta ? delta_dtype : out_dtype;
-  if (dd == CW_F32 && w_dtype == CW_F32 && out_dtype == CW_F32) CW_LAUNCH(float, float, float);
+  const bool vec4 = H % 4 == 0 && dd == CW_BF16 && out_dtype == CW_BF16 &&
+                    (((uintptr_t)resid | (uintptr_t)extra) % 16 == 0) && (((uintptr_t)delta | (uintptr_t)out) % 8 == 0);
+  if (vec4 && w_dtype == CW_BF16)
+    hipLaunchKernelGGL(add_dyt_vec4_kernel<bf16_t>, grid, block, 0, stream, resid, (const bf16_t*)delta, scale, extra,
+                       (const bf16_t*)w, (const bf16_t*)b, alpha, (bf16_t*)out, rows, H);
+  else if (vec4 && w_dtype == CW_F32)
+    hipLaunchKernelGGL(add_dyt_vec4_kernel<float>, grid, block, 0, stream, resid, (const bf16_t*)delta, scale, extra,
+                       (const float*)w, (const float*)b, alpha, (bf16_t*)out, rows, H);
+  else if (dd == CW_F32 && w_dtype == CW_F32 && out_dtype == CW_F32) CW_LAUNCH(float, float, float);
   else if (dd == CW_BF16 && w_dtype == CW_BF16 && out_dtype == CW_BF16) CW_LAUNCH(bf16_t, bf16_t, bf16_t);
   else if (dd == CW_BF16 && w_dtype == CW_F32 && out_dtype == CW_BF16) CW_LAUNCH(bf16_t, float, bf16_t);
   else return CW_ERR_DTYPE;
@@ -388,9 +433,31 @@ __global__ void gelu_erf_kernel(T* __restrict__ x, int64_t n) {
   }
 }
 
+// bfloat16, 8 elements (16 bytes) a thread
+__global__ void gelu_erf_vec8_kernel(uint4* __restrict__ x, int64_t n8) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += (int64_t)gridDim.x * blockDim.x) {
+    uint4 v = x[i];
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float a = cw_bf16_bits_to_float((uint16_t)(w[u] & 0xffffu)), b = cw_bf16_bits_to_float((uint16_t)(w[u] >> 16));
+      const float ga = 0.5f * a * (1.0f + erff(a * 0.70710678118654752440f));
+      const float gb = 0.5f * b * (1.0f + erff(b * 0.70710678118654752440f));
+      w[u] = (uint32_t)cw_float_to_bf16_bits(ga) | ((uint32_t)cw_float_to_bf16_bits(gb) << 16);
+    }
+    x[i] = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
 CW_EXPORT int cw_gelu_erf(void* x, int dtype, int64_t n, hipStream_t stream) {
   if (n < 0) return CW_ERR_ARG;
   if (n == 0) return CW_OK;
+  if (dtype == CW_BF16 && n % 8 == 0 && (uintptr_t)x % 16 == 0) {
+    int64_t blocks8 = (n / 8 + 255) / 256;
+    if (blocks8 > 65536) blocks8 = 65536;
+    hipLaunchKernelGGL(gelu_erf_vec8_kernel, dim3((unsigned)blocks8), dim3(256), 0, stream, (uint4*)x, n / 8);
+    return cw_launch_status();
+  }
   int64_t blocks = (n + 255) / 256;
   if (blocks > 262144) blocks = 262144;
   dim3 grid((unsigned)blocks), block(256);

@@ -46,12 +46,17 @@ def query_runs(ctx, run: int, skip_single: bool = False):
 
 
 def longest_key_range(ctx, window=None, segment=None) -> int:
-    """The most keys that a token of this step reads: its request's length, capped by a window or
-    by the segment's size."""
-    longest = max(ctx.h_ctx_lens, default=0)
-    for cap in (window, segment):
-        if cap is not None:
-            longest = min(longest, cap)
+    """The most keys that a token of this step reads: its request's length, capped by a window;
+    with segments, what the request's last token sees of its own segment (a single token) or at
+    most a whole segment (a portion)."""
+    longest = 0
+    for q_len, ctx_len in zip(ctx.h_q_lens, ctx.h_ctx_lens):
+        keys = ctx_len
+        if window is not None:
+            keys = min(keys, window)
+        if segment is not None:
+            keys = min(keys, segment) if q_len > 1 else (ctx_len - 1) % segment + 1
+        longest = max(longest, keys)
     return longest
 
 
