@@ -91,7 +91,10 @@ def _two_map_sizes(spec):
 # heads, kv_heads, dim, vdim, segment, hidden: grouped heads, a group larger than a workgroup takes
 # at once, sizes of 1, value sizes that are no multiple of 16, a segment longer than the sequence
 TWO_MAP_SHAPES = [(4, 2, 24, 16, 9, 64), (6, 6, 16, 16, 33, 96), (3, 1, 40, 24, 300, 100), (2, 1, 8, 32, 1, 48),
-                  (1, 1, 32, 8, 17, 48), (20, 2, 8, 20, 12, 64), (2, 2, 64, 130, 16, 64), (8, 2, 64, 128, 40, 128)]
+                  (1, 1, 32, 8, 17, 48), (20, 2, 8, 20, 12, 64), (2, 2, 64, 130, 16, 64), (8, 2, 64, 128, 40, 128),
+                  # the other sizes that the matrix-core kernel is built for
+                  (4, 2, 128, 128, 40, 64), (3, 1, 128, 64, 16, 64), (2, 1, 64, 256, 25, 64), (2, 2, 128, 256, 30, 64),
+                  (10, 2, 64, 64, 21, 64)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
