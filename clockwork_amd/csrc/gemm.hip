@@ -197,7 +197,8 @@ CW_EXPORT int cw_gemm_f32(const float* A, int64_t lda, const float* W, const flo
 // operand, loaded from global memory directly in operand layout (lane = row l%16, 8 consecutive
 // k at slot l/16), and 16 tokens x the same k-values as the B operand.
 //
-// MODE 0: y bfloat16 [M, N]; MODE 1: y float32 [M, N] (logits); MODE 2: W is [2I, K] with gate
+// MODE 0: y bfloat16 [M, N]; MODE 4: the same with the erf GELU applied to the float32 sums before
+// they are rounded; MODE 1: y float32 [M, N] (logits); MODE 2: W is [2I, K] with gate
 // rows first, y[m, i] = silu(gate_i) * up_i as bfloat16 [M, I]: a row tile holds 8 gate rows and
 // the 8 up rows that belong to them. MODE 3: K is also split over gridDim.y workgroups, each
 // writing its float32 partial product [split, M, N]; whoever reads y next sums the partials in
@@ -223,6 +224,8 @@ __device__ __forceinline__ bf16x8_t cw_to_operand_layout(const bf16x8_t& v, int 
   for (int d = 0; d < 4; ++d) t[d] = __builtin_amdgcn_ds_bpermute(from, q[d]);
   return __builtin_bit_cast(bf16x8_t, t);
 }
+
+__device__ __forceinline__ float cw_gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f)); }
 
 // ROWS (16, 8 or 4) is the number of weight rows a tile really holds: a narrow output with a long K
 // is cut into more, smaller tiles so that every compute unit streams a share of the matrix (the
@@ -346,6 +349,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
       const float v = red[0][(rt * MT + mt) * 256 + j * 16 + tok];
       if (MODE == 3) ((float*)C)[((int64_t)blockIdx.y * M + m) * ldc + n] = v;
       else if (MODE == 1) ((float*)C)[(int64_t)m * ldc + n] = v;
+      else if (MODE == 4) ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(cw_gelu_erf(v));
       else ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(v);
     }
   }
@@ -512,6 +516,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
         if (m < M && n < N) {
           if (MODE == 3) ((float*)C)[((int64_t)blockIdx.y * M + m) * ldc + n] = v;
           else if (MODE == 1) ((float*)C)[(int64_t)m * ldc + n] = v;
+          else if (MODE == 4) ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(cw_gelu_erf(v));
           else ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(v);
         }
       }
@@ -670,6 +675,7 @@ static int try_stream(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W, v
     case 0: return launch_stream_mt<0, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
     case 1: return launch_stream_mt<1, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
     case 2: return launch_stream_mt<2, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
+    case 4: return launch_stream_mt<4, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
     default: return launch_stream_mt<3, 8>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
   }
 }
@@ -685,6 +691,7 @@ static int launch_skinny(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W
   if (mode == 0) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 0, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
   else if (mode == 1) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 1, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
   else if (mode == 3) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 3, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  else if (mode == 4) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 4, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
   else if (ROWS == 16) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 2, WAVES, 16>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
   else return CW_ERR_ARG;
   return cw_launch_status();
@@ -738,7 +745,7 @@ CW_EXPORT int cw_gemm_bf16_skinny_ksplits(int M, int N, int K) {
 // that range run, but a library product is faster). mode 3 is answered by ..._ksplits() > 1.
 CW_EXPORT int cw_gemm_bf16_skinny_fast(int mode, int M, int N, int K) {
   if (M <= 16) return 1;
-  if (mode < 0 || mode > 2) return 0;
+  if (mode < 0 || (mode > 2 && mode != 4)) return 0;
   int mt, spw, n_tiles;
   dim3 grid;
   return plan_stream(mode, M, N, K, 1, &mt, &spw, &grid, &n_tiles) ? 1 : 0;
@@ -791,7 +798,7 @@ CW_EXPORT int cw_gemm_bf16_swiglu_normed(const float* resid, const void* delta, 
 // cw_gemm_bf16_skinny_ksplits(M, N, K). K must be a multiple of 8 (16-byte rows).
 CW_EXPORT int cw_gemm_bf16_skinny(int mode, const void* X, int64_t ldx, const void* W, void* C,
                                   int64_t ldc, int M, int N, int K, int k_splits, hipStream_t stream) {
-  if (M < 0 || N <= 0 || K <= 0 || mode < 0 || mode > 3) return CW_ERR_ARG;
+  if (M < 0 || N <= 0 || K <= 0 || mode < 0 || mode > 4) return CW_ERR_ARG;
   if (M > CW_SKINNY_MAX_M) return CW_ERR_SIZE;
   if ((K & 7) || (ldx & 7) || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return CW_ERR_ARG;
   if (mode == 2 && (N & 1)) return CW_ERR_ARG;

@@ -1598,6 +1598,23 @@ def add_dynamic_tanh(resid, delta, delta_scale: float, extra, weight, bias, alph
     return out
 
 
+def linear_gelu(x: torch.Tensor, weight: torch.Tensor, policy: "ProductPolicy | None" = None) -> torch.Tensor:
+    """gelu(x @ weight.T), the erf form. Few bfloat16 rows: the weight-streaming product with the
+    activation in its epilogue, applied to the float32 sums (one launch); else the product and the
+    activation kernel."""
+    _gpu(x, weight)
+    M, K = x.shape
+    N = weight.shape[0]
+    if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and weight.shape[1] == K and M <= STREAM_MAX_ROWS
+            and K % 8 == 0):
+        lib = _load("gemm")
+        if lib.cw_gemm_bf16_skinny_fast(4, M, N, K):
+            out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            _check(lib.cw_gemm_bf16_skinny(4, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, 0, _stream()), "gemm_bf16_skinny(gelu)")
+            return out
+    return gelu_erf_(linear(x, weight, policy=policy))
+
+
 def gelu_erf_(x: torch.Tensor) -> torch.Tensor:
     """x <- 0.5 x (1 + erf(x / sqrt 2)), in place."""
     _gpu(x)

@@ -68,8 +68,8 @@ class GatedMLP(Part):
 
 
 class DenseMLP(Part):
-    """down(gelu(up(x))) (``DenseMLPSpec``): the up product, the erf GELU in place (float32
-    inside), the down product."""
+    """down(gelu(up(x))) (``DenseMLPSpec``): the up product with the erf GELU (float32 inside) in
+    its epilogue for few rows, as a kernel of its own behind the product otherwise; the down product."""
 
     graph_safe = True
 
@@ -89,4 +89,4 @@ class DenseMLP(Part):
 
     def forward(self, x, ctx) -> torch.Tensor:
         policy = getattr(ctx, "products", None)
-        return ops.linear(ops.gelu_erf_(ops.linear(x, self.up, policy=policy)), self.down, policy=policy)
+        return ops.linear(ops.linear_gelu(x, self.up, policy=policy), self.down, policy=policy)

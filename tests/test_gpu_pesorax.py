@@ -62,14 +62,21 @@ def test_dynamic_tanh_alone_with_a_scaled_branch_and_with_the_input_again(dtype,
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_dense_gelu_feed_forward(dtype):
+@pytest.mark.parametrize("hidden, rows", [(100, 41), (128, 8), (128, 41), (1024, 3), (128, 200)])
+def test_dense_gelu_feed_forward(dtype, hidden, rows):
+    """Few bfloat16 rows of a width that is a multiple of 8 take the product with the activation
+    in its epilogue, the others the product and the activation kernel."""
     from types import SimpleNamespace
 
-    part = build_part(DenseMLPSpec(hidden_size=100, intermediate_size=72))
+    part = build_part(DenseMLPSpec(hidden_size=hidden, intermediate_size=72))
     w = bind(part, dtype, seed=2, matrix_std=0.2)
-    x = torch.randn(41, 100, generator=torch.Generator().manual_seed(3)).to(dtype)
+    x = torch.randn(rows, hidden, generator=torch.Generator().manual_seed(3)).to(dtype)
     got = part.forward(x.to(DEV), SimpleNamespace()).double().cpu()
     close(got, plain.dense_feed_forward(x.double(), {"up": w["up_weight"], "down": w["down_weight"]}, ""), dtype)
+    if dtype == torch.bfloat16:
+        inner = ops.linear_gelu(x.to(DEV), part.up).double().cpu()
+        want = plain.gelu_erf(x.double() @ w["up_weight"].t())
+        close(inner, want, dtype)
 
 
 # ------------------------------------------------------------------------------- two-map attention
